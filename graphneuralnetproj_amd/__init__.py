@@ -1,0 +1,13 @@
+"""MI355X-native Tiled-CSL SpMM: Python mirror of the C ABI in include/SpMM_API.h."""
+from .spmm_api import (  # noqa: F401
+    GenSparseMatrixBinFile,
+    InitSparseMatrixA_API,
+    SpMM_SplitK_API,
+    SpMM_SuggestSplitK,
+    SpMMError,
+    build_library,
+    library_path,
+    load_library,
+    synth_activations,
+    synth_weights,
+)

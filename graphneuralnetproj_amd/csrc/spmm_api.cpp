@@ -1,0 +1,108 @@
+// Host logic behind the C ABI declared in include/SpMM_API.h: argument
+// checking, the split-K plan and the order of launches.  Plain C++; the GPU is
+// reached only through the tcsl_* launchers of spmm_kernels.hip.
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+
+#include "../../include/SpMM_API.h"
+#include "tiled_csl_format.h"
+
+extern "C" {
+int tcsl_launch_spmm(void* stream, const void* items, const int* offsets, const void* B, void* out, int M, int N,
+                     int K, int split_k);
+int tcsl_launch_reduce(void* stream, void* C, const void* W, long mn, int split_k);
+int tcsl_launch_copy(void* stream, void* dst, const void* src, long bytes);
+const char* tcsl_error_string(int code);
+int tcsl_error_unknown(void);
+int tcsl_error_invalid_value(void);
+}
+
+extern "C" int InitSparseMatrixA_API(const uint16_t* A_h, int M, int N, int K, uint32_t** Compressed_A,
+                                     int** TileOffsets)
+{
+    (void)N;  // unused by the reference too (csrc/SpMM_API.cu:241-246)
+    return tcsl::encode(A_h, M, K, Compressed_A, TileOffsets);
+}
+
+extern "C" int GenSparseMatrixBinFile(char* DenseMatrixFileName, int M, int K, char* NZWeightsFileName,
+                                      char* TileOffsetsFileName, char* OutputSizesFileName)
+{
+    return tcsl::encode_file(DenseMatrixFileName, M, K, NZWeightsFileName, TileOffsetsFileName, OutputSizesFileName);
+}
+
+extern "C" void SpMM_FreeHost(void* p)
+{
+    std::free(p);
+}
+
+extern "C" const char* SpMM_GetErrorString(int code)
+{
+    return tcsl_error_string(code);
+}
+
+extern "C" int SpMM_SplitK_API(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets,
+                               const void* B, void* C, int M, int N, int K, void* Reduction_Workspace, int Split_K)
+{
+    (void)A;
+    if (N != 8 && N != 16 && N != 32 && N != 64) {
+        std::printf("MM_Sparse_API Error: Unsupported N dimension %d!\n", N);
+        return tcsl_error_unknown();
+    }
+    if (M <= 0 || K <= 0 || M % tcsl::kTileRows != 0 || K % tcsl::kTileCols != 0 || Split_K < 1) {
+        std::fprintf(stderr, "SpMM_SplitK_API: unsupported shape M=%d K=%d Split_K=%d (need M %% 128 == 0, K %% 64 == 0, Split_K >= 1)\n",
+                     M, K, Split_K);
+        return tcsl_error_invalid_value();
+    }
+    if (!Compressed_A || !TileOffsets || !B || !C || (Split_K > 1 && !Reduction_Workspace)) {
+        std::fprintf(stderr, "SpMM_SplitK_API: null device pointer\n");
+        return tcsl_error_invalid_value();
+    }
+    // the launch grid is (M/128) * Split_K single-wave workgroups
+    if (static_cast<long>(M / tcsl::kTileRows) * Split_K > 0x7fffffffL) {
+        std::fprintf(stderr, "SpMM_SplitK_API: Split_K=%d too large for M=%d\n", Split_K, M);
+        return tcsl_error_invalid_value();
+    }
+    if (Split_K == 1)
+        return tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, C, M, N, K, 1);
+    int rc = tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, Reduction_Workspace, M, N, K, Split_K);
+    if (rc != 0)
+        return rc;
+    return tcsl_launch_reduce(stream, C, Reduction_Workspace, static_cast<long>(M) * N, Split_K);
+}
+
+extern "C" int SpMM_SuggestSplitK(int M, int N, int K)
+{
+    (void)N;
+    if (M <= 0 || K <= 0)
+        return 1;
+    // One wave per (128-row tile row, batch); a compute unit holds up to ten of
+    // them (LDS bound), and seven to eight per unit keep enough loads in flight.
+    const long row_tiles = (M + tcsl::kTileRows - 1) / tcsl::kTileRows;
+    const long nkb = K / tcsl::kTileCols > 0 ? K / tcsl::kTileCols : 1;
+    const long target_waves = 256L * 8;
+    long s = (target_waves + row_tiles - 1) / row_tiles;
+    const long max_split = nkb / 4 > 0 ? nkb / 4 : 1;  // at least four tiles per batch
+    if (s > max_split)
+        s = max_split;
+    if (s < 1)
+        s = 1;
+    return static_cast<int>(s);
+}
+
+extern "C" void SpMM_SynthWeights(uint16_t* A_h, int M, int K, double sparsity, int row_skewed, uint64_t seed)
+{
+    tcsl::synth_weights(A_h, M, K, sparsity, row_skewed, seed);
+}
+
+extern "C" void SpMM_SynthActivations(uint16_t* B_h, long count, uint64_t seed)
+{
+    tcsl::synth_activations(B_h, count, seed);
+}
+
+extern "C" int SpMM_CalibrationCopy(void* stream, void* dst, const void* src, long bytes)
+{
+    if (!dst || !src || bytes < 0 || bytes % 16 != 0)
+        return tcsl_error_invalid_value();
+    return tcsl_launch_copy(stream, dst, src, bytes);
+}

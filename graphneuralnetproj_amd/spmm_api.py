@@ -1,0 +1,192 @@
+"""ctypes mirror of libSpMM_API.so, with the reference's names and argument order.
+
+The functions here add nothing to the C ABI: they convert numpy arrays and
+device pointers, call through, and turn error codes into exceptions.  There is
+no CPU fallback: if the library has not been built, loading fails.
+
+Reference interfaces mirrored (paths relative to the reference checkout):
+  InitSparseMatrixA_API   build/SpMM_API.cuh:55, csrc/SpMM_API.cu:241-438
+  SpMM_SplitK_API         third_party/ft.patch:2833-2843, csrc/SpMM_API.cu:79-208
+  GenSparseMatrixBinFile  csrc/SpMM_API.cu:1565-1620,
+                          end2end_inference/ft_tools/huggingface_opt_convert_Phase2.py:36-59
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_PKG, "lib", "libSpMM_API.so")
+
+_u16p = ctypes.POINTER(ctypes.c_uint16)
+_u32p = ctypes.POINTER(ctypes.c_uint32)
+_i32p = ctypes.POINTER(ctypes.c_int)
+
+EXPORTED_SYMBOLS = (
+    "InitSparseMatrixA_API",
+    "SpMM_SplitK_API",
+    "GenSparseMatrixBinFile",
+    "SpMM_FreeHost",
+    "SpMM_GetErrorString",
+    "SpMM_SuggestSplitK",
+    "SpMM_SynthWeights",
+    "SpMM_SynthActivations",
+    "SpMM_CalibrationCopy",
+)
+
+
+class SpMMError(RuntimeError):
+    """A non-zero code from the library."""
+
+    def __init__(self, where, code, text=""):
+        super().__init__(f"{where} failed with code {code}" + (f" ({text})" if text else ""))
+        self.code = code
+
+
+def library_path():
+    return _LIB_PATH
+
+
+def build_library():
+    """Compile the library in-tree with hipcc (always recompiles)."""
+    csrc = os.path.join(_PKG, "csrc")
+    subprocess.run(["make", "-s", "-C", csrc, "clean"], check=True)
+    subprocess.run(["make", "-s", "-C", csrc, "-j4"], check=True)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def load_library():
+    """Load libSpMM_API.so; raises if it is missing (no fallback)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise FileNotFoundError(
+            f"{_LIB_PATH} not found: build it with graphneuralnetproj_amd.build_library() "
+            "or `make -C graphneuralnetproj_amd/csrc`")
+    # A process must hold ONE HIP runtime.  Device memory and streams come from
+    # PyTorch here, and PyTorch ships its own libamdhip64 (same soname as the
+    # system one): importing it first makes the loader bind this library to that
+    # copy instead of mapping a second runtime that cannot see the device.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
+    lib = ctypes.CDLL(_LIB_PATH)
+    lib.InitSparseMatrixA_API.restype = ctypes.c_int
+    lib.InitSparseMatrixA_API.argtypes = [_u16p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(_u32p),
+                                          ctypes.POINTER(_i32p)]
+    lib.SpMM_SplitK_API.restype = ctypes.c_int
+    lib.SpMM_SplitK_API.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_int]
+    lib.GenSparseMatrixBinFile.restype = ctypes.c_int
+    lib.GenSparseMatrixBinFile.argtypes = [ctypes.c_char_p, ctypes.c_int, ctypes.c_int, ctypes.c_char_p,
+                                           ctypes.c_char_p, ctypes.c_char_p]
+    lib.SpMM_FreeHost.restype = None
+    lib.SpMM_FreeHost.argtypes = [ctypes.c_void_p]
+    lib.SpMM_GetErrorString.restype = ctypes.c_char_p
+    lib.SpMM_GetErrorString.argtypes = [ctypes.c_int]
+    lib.SpMM_SuggestSplitK.restype = ctypes.c_int
+    lib.SpMM_SuggestSplitK.argtypes = [ctypes.c_int] * 3
+    lib.SpMM_SynthWeights.restype = None
+    lib.SpMM_SynthWeights.argtypes = [_u16p, ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_int,
+                                      ctypes.c_uint64]
+    lib.SpMM_SynthActivations.restype = None
+    lib.SpMM_SynthActivations.argtypes = [_u16p, ctypes.c_long, ctypes.c_uint64]
+    lib.SpMM_CalibrationCopy.restype = ctypes.c_int
+    lib.SpMM_CalibrationCopy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_long]
+    _lib = lib
+    return lib
+
+
+def _bits(a):
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.float16:
+        return a.view(np.uint16)
+    if a.dtype != np.uint16:
+        raise TypeError(f"expected float16 (or uint16 bit patterns), got {a.dtype}")
+    return a
+
+
+def InitSparseMatrixA_API(A_h, M=None, N=0, K=None):
+    """Encode a row-major fp16 M x K host matrix.
+
+    Returns (Compressed_A uint32[4*TileOffsets[-1]], TileOffsets int32[(M/128)*(K/64)+2]);
+    len(TileOffsets) is what the C function returns.  Raises SpMMError on a
+    shape the reference would assert on.
+    """
+    a = _bits(A_h)
+    if M is None or K is None:
+        M, K = a.shape
+    if a.size != M * K:
+        raise ValueError(f"A_h has {a.size} elements, expected {M}*{K}")
+    lib = load_library()
+    items, offs = _u32p(), _i32p()
+    n = lib.InitSparseMatrixA_API(a.ctypes.data_as(_u16p), M, N, K, ctypes.byref(items), ctypes.byref(offs))
+    if n < 0:
+        raise SpMMError("InitSparseMatrixA_API", n)
+    offsets = np.ctypeslib.as_array(offs, shape=(n,)).astype(np.int32, copy=True)
+    nwords = int(offsets[-1]) * 4
+    compressed = (np.ctypeslib.as_array(items, shape=(nwords,)).astype(np.uint32, copy=True)
+                  if nwords else np.zeros(0, dtype=np.uint32))
+    lib.SpMM_FreeHost(items)
+    lib.SpMM_FreeHost(offs)
+    return compressed, offsets
+
+
+def _ptr(x):
+    """Device pointer of a torch tensor, or a raw integer address, or None."""
+    if x is None:
+        return None
+    if isinstance(x, int):
+        return ctypes.c_void_p(x)
+    return ctypes.c_void_p(x.data_ptr())
+
+
+def SpMM_SplitK_API(stream, A, Compressed_A, TileOffsets, B, C, M_Global, N_Global, K_Global, Reduction_Workspace,
+                    Split_K):
+    """Enqueue C = A * B on `stream` (an integer hipStream_t or a torch stream; None = default).
+
+    Tensor arguments are torch CUDA tensors (or raw device addresses); A is
+    unused and may be None.  Returns 0; raises SpMMError with the hipError_t
+    code otherwise.
+    """
+    lib = load_library()
+    if stream is not None and not isinstance(stream, int):
+        stream = stream.cuda_stream
+    rc = lib.SpMM_SplitK_API(ctypes.c_void_p(stream) if stream else None, _ptr(A), _ptr(Compressed_A),
+                             _ptr(TileOffsets), _ptr(B), _ptr(C), M_Global, N_Global, K_Global,
+                             _ptr(Reduction_Workspace), Split_K)
+    if rc != 0:
+        raise SpMMError("SpMM_SplitK_API", rc, lib.SpMM_GetErrorString(rc).decode())
+    return rc
+
+
+def GenSparseMatrixBinFile(DenseMatrixFileName, M, K, NZWeightsFileName, TileOffsetsFileName, OutputSizesFileName):
+    lib = load_library()
+    rc = lib.GenSparseMatrixBinFile(DenseMatrixFileName.encode(), M, K, NZWeightsFileName.encode(),
+                                    TileOffsetsFileName.encode(), OutputSizesFileName.encode())
+    if rc != 0:
+        raise SpMMError("GenSparseMatrixBinFile", rc)
+    return rc
+
+
+def SpMM_SuggestSplitK(M_Global, N_Global, K_Global):
+    return load_library().SpMM_SuggestSplitK(M_Global, N_Global, K_Global)
+
+
+def synth_weights(M, K, sparsity, row_skewed=False, seed=0):
+    """Deterministic synthetic fp16 weight, row-major M x K."""
+    A = np.empty((M, K), dtype=np.uint16)
+    load_library().SpMM_SynthWeights(A.ctypes.data_as(_u16p), M, K, float(sparsity), int(bool(row_skewed)), seed)
+    return A.view(np.float16)
+
+
+def synth_activations(N, K, seed=0):
+    """Deterministic synthetic fp16 activations, one K vector per token (N x K)."""
+    B = np.empty((N, K), dtype=np.uint16)
+    load_library().SpMM_SynthActivations(B.ctypes.data_as(_u16p), N * K, seed)
+    return B.view(np.float16)

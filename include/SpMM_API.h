@@ -1,0 +1,123 @@
+/*
+ * libSpMM_API.so -- MI355X (gfx950) implementation of the Tiled-CSL sparse
+ * weight x dense activation product.  Plain C ABI: every symbol is extern "C",
+ * arguments are raw pointers and ints, no HIP or torch types appear.
+ *
+ * Each entry point names the reference interface it stands in for (paths are
+ * relative to the reference checkout).  The reference's own symbols are C++
+ * (mangled) except GenSparseMatrixBinFile; here all of them are C symbols with
+ * the same names and the same argument order.
+ *
+ * Data layout
+ *   A            row-major M x K fp16 (A[m*K + k]); only read by the encoder.
+ *   Compressed_A packed words, one per kept element plus zero padding to a
+ *                multiple of 4 per 128x64 tile: bits 0-15 fp16 value, bits 16-31
+ *                row*64 + (col ^ ((row % 8) << 3)) within the tile.
+ *   TileOffsets  (M/128)*(K/64) + 2 ints, in units of 4 words; tile t (row-major
+ *                over tiles) owns words [4*TileOffsets[t], 4*TileOffsets[t+1]);
+ *                the last two entries are equal.
+ *   B            activations, one contiguous K vector per token:  B[n*K + k].
+ *   C            result, one contiguous M vector per token:       C[n*M + m].
+ *                (the column-major convention of csrc/MatMulUtilities.cuh:15-18,
+ *                the one the FasterTransformer caller uses, third_party/ft.patch:2823-2846)
+ */
+#ifndef TILED_CSL_SPMM_API_H
+#define TILED_CSL_SPMM_API_H
+
+#include <stdint.h>
+
+#define SPMM_EXPORT __attribute__((visibility("default")))
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/*
+ * Host encoder.  Stands in for
+ *   int InitSparseMatrixA_API(half* A_h, int M, int N, int K, uint32_t** Compressed_A, int** TileOffsets)
+ *   (declared build/SpMM_API.cuh:55, defined csrc/SpMM_API.cu:241-438).
+ * A_h holds fp16 bit patterns; N is ignored, as in the reference.  On success
+ * *Compressed_A and *TileOffsets are malloc()ed (the caller frees them, with
+ * free() or SpMM_FreeHost) and the number of TileOffsets entries is returned;
+ * the word count is 4 * (*TileOffsets)[ret - 1].  Output is bit-identical to the
+ * reference's.  Where the reference asserts or exits, a negative code comes back
+ * and nothing is allocated:  -1 M % 128 or K % 64 != 0 (or not positive),
+ * -2 out of memory, -3 null pointer, -5 more than 2^31-1 vectors.
+ * Re-entrant.  Uses up to 16 host threads (SPMM_ENCODE_THREADS overrides).
+ */
+SPMM_EXPORT int InitSparseMatrixA_API(const uint16_t* A_h, int M, int N, int K, uint32_t** Compressed_A, int** TileOffsets);
+
+/*
+ * The product C = A * B on the GPU.  Stands in for
+ *   cudaError_t SpMM_SplitK_API(cudaStream_t stream, const half* A, const uint4* Compressed_A,
+ *                               const int* TileOffsets, const half* B, half* C,
+ *                               int M_Global, int N_Global, int K_Global,
+ *                               half* Reduction_Workspace, int Split_K)
+ *   in the 11-argument form its caller uses (third_party/ft.patch:2833-2843; this
+ *   checkout's declaration, build/SpMM_API.cuh:40-52, carries two extra operands of
+ *   an unrelated format; dispatch and semantics csrc/SpMM_API.cu:79-208).
+ * stream is a hipStream_t (NULL = the default stream).  A is unused and may be
+ * NULL.  All other pointers are device memory owned by the caller.  The call
+ * only enqueues work on `stream`; it never synchronises.
+ *   Split_K == 1: C is written directly, the workspace is not touched.
+ *   Split_K  > 1: batch b of ceil((K/64)/Split_K) column tiles writes fp16 partial
+ *                 sums to Reduction_Workspace[b*M*N ..), then C = fp16(sum in fp32).
+ *                 Reduction_Workspace must hold Split_K*M*N fp16 values and may be
+ *                 shared by successive calls on one stream.
+ * Accumulation is fp32.  Returns the hipError_t value: 0 on success;
+ * hipErrorUnknown, after printing the reference's message, for N outside
+ * {8, 16, 32, 64} (csrc/SpMM_API.cu:192-193); hipErrorInvalidValue for M % 128,
+ * K % 64, Split_K < 1 or a null pointer (the reference checks these only in
+ * debug builds, :93-98, and requires M % 256).  Nothing is launched on error.
+ * Thread safe: no mutable state.
+ */
+SPMM_EXPORT int SpMM_SplitK_API(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets, const void* B,
+                    void* C, int M_Global, int N_Global, int K_Global, void* Reduction_Workspace, int Split_K);
+
+/*
+ * File-to-file encoder used by model converters.  Stands in for
+ *   extern "C" void GenSparseMatrixBinFile(char* DenseMatrixFileName, int M, int K,
+ *                                          char* NZWeightsFileName, char* TileOffsetsFileName,
+ *                                          char* OutputSizesFileName)
+ *   (defined csrc/SpMM_API.cu:1565-1620; called through ctypes by
+ *   end2end_inference/ft_tools/huggingface_opt_convert_Phase2.py:36-59).
+ * Reads M*K fp16 values, writes the packed words (uint32), the offsets (int32)
+ * and two int32 {word count, number of offsets}.  Returns 0, or a negative code
+ * (-4 file error, otherwise as InitSparseMatrixA_API) where the reference exits.
+ */
+SPMM_EXPORT int GenSparseMatrixBinFile(char* DenseMatrixFileName, int M, int K, char* NZWeightsFileName,
+                           char* TileOffsetsFileName, char* OutputSizesFileName);
+
+/* free() for buffers returned by InitSparseMatrixA_API (for callers without a C runtime at hand). */
+SPMM_EXPORT void SpMM_FreeHost(void* p);
+
+/* Text for a code returned by SpMM_SplitK_API. */
+SPMM_EXPORT const char* SpMM_GetErrorString(int code);
+
+/*
+ * A Split_K that fills the 256 compute units of an MI355X for this shape; the
+ * counterpart of the reference's hand-tuned per-shape table
+ * (kernel_benchmark/benchmark.sh:15, huggingface_opt_convert_Phase2.py:20).
+ */
+SPMM_EXPORT int SpMM_SuggestSplitK(int M_Global, int N_Global, int K_Global);
+
+/*
+ * Deterministic synthetic inputs for tests and benchmarks (host memory, fp16 bit
+ * patterns): Bernoulli or Beta(2,8)-row-skewed sparsity with N(0, 0.02) weights,
+ * N(0, 1) activations.  No counterpart in the reference, whose harness uses
+ * unseeded rand() (kernel_benchmark/spmm_test_utils.h:108-141).
+ */
+SPMM_EXPORT void SpMM_SynthWeights(uint16_t* A_h, int M, int K, double sparsity, int row_skewed, uint64_t seed);
+SPMM_EXPORT void SpMM_SynthActivations(uint16_t* B_h, long count, uint64_t seed);
+
+/*
+ * Device-to-device streaming copy of `bytes` (multiple of 16) on `stream`; a
+ * transfer of known size against which hardware byte counters are calibrated.
+ * No counterpart in the reference.
+ */
+SPMM_EXPORT int SpMM_CalibrationCopy(void* stream, void* dst, const void* src, long bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,165 @@
+"""TEST INFRASTRUCTURE ONLY: ctypes doors onto the CPU checkers.
+
+``liboracle.so`` is the C restatement (``tiled_csl_oracle.c``);
+``_ref/libref_encoder.so`` is the reference's own host encoder compiled by
+``oracle/Makefile`` (present only where that build ran).  Only tests,
+``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may
+import this module; the product never does.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_ORACLE_SO = os.path.join(_HERE, "liboracle.so")
+_REF_SO = os.path.join(_HERE, "_ref", "libref_encoder.so")
+
+_u16p = ctypes.POINTER(ctypes.c_uint16)
+_u32p = ctypes.POINTER(ctypes.c_uint32)
+_i32p = ctypes.POINTER(ctypes.c_int)
+_f32p = ctypes.POINTER(ctypes.c_float)
+
+
+def build(with_ref=True):
+    """(Re)build the checkers with oracle/Makefile."""
+    targets = ["oracle"] + (["ref"] if with_ref else [])
+    subprocess.run(["make", "-s", "-C", _HERE] + targets, check=True)
+
+
+def _load():
+    if not os.path.exists(_ORACLE_SO):
+        build(with_ref=False)
+    lib = ctypes.CDLL(_ORACLE_SO)
+    lib.oracle_half_to_float.restype = ctypes.c_float
+    lib.oracle_half_to_float.argtypes = [ctypes.c_uint16]
+    lib.oracle_float_to_half_rn.restype = ctypes.c_uint16
+    lib.oracle_float_to_half_rn.argtypes = [ctypes.c_float]
+    lib.oracle_encode.restype = ctypes.c_int
+    lib.oracle_encode.argtypes = [_u16p, ctypes.c_int, ctypes.c_int, ctypes.POINTER(_u32p), ctypes.POINTER(_i32p)]
+    lib.oracle_free.argtypes = [ctypes.c_void_p]
+    lib.oracle_decode.argtypes = [_u32p, _i32p, ctypes.c_int, ctypes.c_int, _u16p]
+    lib.oracle_gemm_f32.argtypes = [_u16p, _u16p, _f32p] + [ctypes.c_int] * 5
+    lib.oracle_splitk_range.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, _i32p, _i32p]
+    lib.oracle_reduce.argtypes = [_u16p, _u16p, ctypes.c_long, ctypes.c_int]
+    lib.oracle_spmm_splitk.restype = ctypes.c_int
+    lib.oracle_spmm_splitk.argtypes = [_u32p, _i32p, _u16p, _u16p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u16p,
+                                       ctypes.c_int]
+    return lib
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        _lib = _load()
+    return _lib
+
+
+def _bits(a):
+    """fp16 array (or uint16 bit array) -> contiguous uint16 view."""
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.float16:
+        return a.view(np.uint16)
+    assert a.dtype == np.uint16, a.dtype
+    return a
+
+
+def _take(ptr, n, dtype, free):
+    out = np.ctypeslib.as_array(ptr, shape=(max(n, 1),))[:n].astype(dtype, copy=True)
+    free(ptr)
+    return out
+
+
+def encode(A):
+    """Oracle Tiled-CSL encode of a row-major fp16 M x K matrix -> (items u32, offsets i32)."""
+    M, K = A.shape
+    a = _bits(A)
+    items, offs = _u32p(), _i32p()
+    n = lib().oracle_encode(a.ctypes.data_as(_u16p), M, K, ctypes.byref(items), ctypes.byref(offs))
+    if n < 0:
+        raise ValueError(f"oracle_encode failed with {n} for M={M} K={K}")
+    o = np.ctypeslib.as_array(offs, shape=(n,)).astype(np.int32, copy=True)
+    it = _take(items, int(o[-1]) * 4, np.uint32, lib().oracle_free)
+    lib().oracle_free(offs)
+    return it, o
+
+
+def decode(items, offsets, M, K):
+    items = np.ascontiguousarray(items, dtype=np.uint32)
+    offsets = np.ascontiguousarray(offsets, dtype=np.int32)
+    out = np.empty((M, K), dtype=np.uint16)
+    lib().oracle_decode(items.ctypes.data_as(_u32p), offsets.ctypes.data_as(_i32p), M, K, out.ctypes.data_as(_u16p))
+    return out.view(np.float16)
+
+
+def gemm_f32(A, B, k_begin=0, k_end=None):
+    """A: M x K fp16 row-major; B: N x K fp16 (one K-vector per token) -> C: N x M fp32."""
+    M, K = A.shape
+    N = B.shape[0]
+    assert B.shape[1] == K
+    a, b = _bits(A), _bits(B)
+    C = np.empty((N, M), dtype=np.float32)
+    lib().oracle_gemm_f32(a.ctypes.data_as(_u16p), b.ctypes.data_as(_u16p), C.ctypes.data_as(_f32p), M, N, K, k_begin,
+                          K if k_end is None else k_end)
+    return C
+
+
+def splitk_range(K, split_k, b):
+    s, e = ctypes.c_int(), ctypes.c_int()
+    lib().oracle_splitk_range(K, split_k, b, ctypes.byref(s), ctypes.byref(e))
+    return s.value, e.value
+
+
+def reduce(W, MN, split_k):
+    w = _bits(W).reshape(-1)
+    C = np.empty(MN, dtype=np.uint16)
+    lib().oracle_reduce(C.ctypes.data_as(_u16p), w.ctypes.data_as(_u16p), MN, split_k)
+    return C.view(np.float16)
+
+
+def spmm_splitk(items, offsets, B, M, N, K, split_k):
+    """Whole call on the CPU -> (C fp16 N x M, workspace fp16 split_k x N x M)."""
+    items = np.ascontiguousarray(items, dtype=np.uint32)
+    offsets = np.ascontiguousarray(offsets, dtype=np.int32)
+    b = _bits(B)
+    C = np.zeros((N, M), dtype=np.uint16)
+    W = np.zeros((split_k, N, M), dtype=np.uint16)
+    rc = lib().oracle_spmm_splitk(items.ctypes.data_as(_u32p), offsets.ctypes.data_as(_i32p), b.ctypes.data_as(_u16p),
+                                  C.ctypes.data_as(_u16p), M, N, K, W.ctypes.data_as(_u16p), split_k)
+    if rc:
+        raise ValueError(f"oracle_spmm_splitk rejected M={M} N={N} K={K} split_k={split_k}")
+    return C.view(np.float16), W.view(np.float16)
+
+
+# ----------------------------------------------------------------------------
+# the reference's own encoder, where oracle/_ref was built
+
+
+def have_ref():
+    return os.path.exists(_REF_SO)
+
+
+_ref = None
+
+
+def ref_encode(A):
+    """Encode with the reference's InitSparseMatrixA_API (csrc/SpMM_API.cu:241-438)."""
+    global _ref
+    if _ref is None:
+        _ref = ctypes.CDLL(_REF_SO)
+        _ref.ref_InitSparseMatrixA_API.restype = ctypes.c_int
+        _ref.ref_InitSparseMatrixA_API.argtypes = [_u16p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                   ctypes.POINTER(_u32p), ctypes.POINTER(_i32p)]
+        _ref.ref_free.argtypes = [ctypes.c_void_p]
+    M, K = A.shape
+    a = _bits(A).copy()
+    items, offs = _u32p(), _i32p()
+    n = _ref.ref_InitSparseMatrixA_API(a.ctypes.data_as(_u16p), M, 0, K, ctypes.byref(items), ctypes.byref(offs))
+    o = np.ctypeslib.as_array(offs, shape=(n,)).astype(np.int32, copy=True)
+    it = _take(items, int(o[-1]) * 4, np.uint32, _ref.ref_free)
+    _ref.ref_free(offs)
+    return it, o
