@@ -13,6 +13,10 @@ int tcsl_launch_spmm(void* stream, const void* items, const int* offsets, const 
                      int K, int split_k);
 int tcsl_launch_reduce(void* stream, void* C, const void* W, long mn, int split_k);
 int tcsl_launch_copy(void* stream, void* dst, const void* src, long bytes);
+void* tcsl_event_create(void);
+void tcsl_event_destroy(void* e);
+int tcsl_event_record(void* e, void* stream);
+float tcsl_event_elapsed_ms(void* start, void* stop);
 const char* tcsl_error_string(int code);
 int tcsl_error_unknown(void);
 int tcsl_error_invalid_value(void);
@@ -41,10 +45,52 @@ extern "C" const char* SpMM_GetErrorString(int code)
     return tcsl_error_string(code);
 }
 
+namespace {
+int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* C, int M, int N,
+                int K, void* Reduction_Workspace, int Split_K, void* ev_begin, void* ev_end);
+}
+
 extern "C" int SpMM_SplitK_API(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets,
                                const void* B, void* C, int M, int N, int K, void* Reduction_Workspace, int Split_K)
 {
     (void)A;
+    return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, nullptr,
+                       nullptr);
+}
+
+extern "C" int SpMM_SplitK_API_Events(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets,
+                                      const void* B, void* C, int M, int N, int K, void* Reduction_Workspace,
+                                      int Split_K, void* KernelBegin, void* KernelEnd)
+{
+    (void)A;
+    return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, KernelBegin,
+                       KernelEnd);
+}
+
+extern "C" void* SpMM_EventCreate(void)
+{
+    return tcsl_event_create();
+}
+
+extern "C" void SpMM_EventDestroy(void* event)
+{
+    tcsl_event_destroy(event);
+}
+
+extern "C" int SpMM_EventRecord(void* event, void* stream)
+{
+    return event ? tcsl_event_record(event, stream) : tcsl_error_invalid_value();
+}
+
+extern "C" float SpMM_EventElapsedMs(void* start, void* stop)
+{
+    return (start && stop) ? tcsl_event_elapsed_ms(start, stop) : -1.f;
+}
+
+namespace {
+int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* C, int M, int N,
+                int K, void* Reduction_Workspace, int Split_K, void* ev_begin, void* ev_end)
+{
     if (N != 8 && N != 16 && N != 32 && N != 64) {
         std::printf("MM_Sparse_API Error: Unsupported N dimension %d!\n", N);
         return tcsl_error_unknown();
@@ -63,13 +109,21 @@ extern "C" int SpMM_SplitK_API(void* stream, const void* A, const void* Compress
         std::fprintf(stderr, "SpMM_SplitK_API: Split_K=%d too large for M=%d\n", Split_K, M);
         return tcsl_error_invalid_value();
     }
-    if (Split_K == 1)
-        return tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, C, M, N, K, 1);
-    int rc = tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, Reduction_Workspace, M, N, K, Split_K);
+    // optional events bracket the main kernel only (not the reduction)
+    int rc = 0;
+    if (ev_begin && (rc = tcsl_event_record(ev_begin, stream)) != 0)
+        return rc;
+    rc = tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, Split_K == 1 ? C : Reduction_Workspace, M, N, K,
+                          Split_K);
     if (rc != 0)
         return rc;
+    if (ev_end && (rc = tcsl_event_record(ev_end, stream)) != 0)
+        return rc;
+    if (Split_K == 1)
+        return 0;
     return tcsl_launch_reduce(stream, C, Reduction_Workspace, static_cast<long>(M) * N, Split_K);
 }
+}  // namespace
 
 extern "C" int SpMM_SuggestSplitK(int M, int N, int K)
 {

@@ -314,6 +314,35 @@ extern "C" int tcsl_launch_copy(void* stream, void* dst, const void* src, long b
     return static_cast<int>(hipGetLastError());
 }
 
+// Timing events for benchmarks (the host logic never includes HIP headers).
+extern "C" void* tcsl_event_create(void)
+{
+    hipEvent_t e = nullptr;
+    return hipEventCreate(&e) == hipSuccess ? static_cast<void*>(e) : nullptr;
+}
+
+extern "C" void tcsl_event_destroy(void* e)
+{
+    if (e)
+        (void)hipEventDestroy(static_cast<hipEvent_t>(e));
+}
+
+extern "C" int tcsl_event_record(void* e, void* stream)
+{
+    return static_cast<int>(hipEventRecord(static_cast<hipEvent_t>(e), static_cast<hipStream_t>(stream)));
+}
+
+// Waits for `stop`, then returns stop - start in milliseconds (negative on error).
+extern "C" float tcsl_event_elapsed_ms(void* start, void* stop)
+{
+    float ms = -1.f;
+    if (hipEventSynchronize(static_cast<hipEvent_t>(stop)) != hipSuccess)
+        return -1.f;
+    if (hipEventElapsedTime(&ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)) != hipSuccess)
+        return -1.f;
+    return ms;
+}
+
 extern "C" const char* tcsl_error_string(int code)
 {
     return hipGetErrorString(static_cast<hipError_t>(code));

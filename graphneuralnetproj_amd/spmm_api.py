@@ -33,6 +33,11 @@ EXPORTED_SYMBOLS = (
     "SpMM_SynthWeights",
     "SpMM_SynthActivations",
     "SpMM_CalibrationCopy",
+    "SpMM_SplitK_API_Events",
+    "SpMM_EventCreate",
+    "SpMM_EventDestroy",
+    "SpMM_EventRecord",
+    "SpMM_EventElapsedMs",
 )
 
 
@@ -98,6 +103,16 @@ def load_library():
     lib.SpMM_SynthActivations.argtypes = [_u16p, ctypes.c_long, ctypes.c_uint64]
     lib.SpMM_CalibrationCopy.restype = ctypes.c_int
     lib.SpMM_CalibrationCopy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_long]
+    lib.SpMM_SplitK_API_Events.restype = ctypes.c_int
+    lib.SpMM_SplitK_API_Events.argtypes = lib.SpMM_SplitK_API.argtypes + [ctypes.c_void_p, ctypes.c_void_p]
+    lib.SpMM_EventCreate.restype = ctypes.c_void_p
+    lib.SpMM_EventCreate.argtypes = []
+    lib.SpMM_EventDestroy.restype = None
+    lib.SpMM_EventDestroy.argtypes = [ctypes.c_void_p]
+    lib.SpMM_EventRecord.restype = ctypes.c_int
+    lib.SpMM_EventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+    lib.SpMM_EventElapsedMs.restype = ctypes.c_float
+    lib.SpMM_EventElapsedMs.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
     _lib = lib
     return lib
 

@@ -75,6 +75,23 @@ SPMM_EXPORT int SpMM_SplitK_API(void* stream, const void* A, const void* Compres
                     void* C, int M_Global, int N_Global, int K_Global, void* Reduction_Workspace, int Split_K);
 
 /*
+ * SpMM_SplitK_API with two hipEvent_t recorded on `stream` immediately before and
+ * after the main kernel (the split-K reduction, if any, follows KernelEnd), so a
+ * benchmark can time that kernel alone inside its own loop.  Either event may be
+ * NULL.  The SpMM_Event* helpers create and read such events without HIP headers.
+ * No counterpart in the reference, whose harness times whole calls with cudaEvents
+ * (kernel_benchmark/spmm_test.cu:467-561).
+ */
+SPMM_EXPORT int SpMM_SplitK_API_Events(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets,
+                                       const void* B, void* C, int M_Global, int N_Global, int K_Global,
+                                       void* Reduction_Workspace, int Split_K, void* KernelBegin, void* KernelEnd);
+SPMM_EXPORT void* SpMM_EventCreate(void);
+SPMM_EXPORT void SpMM_EventDestroy(void* event);
+SPMM_EXPORT int SpMM_EventRecord(void* event, void* stream);
+/* Waits for `stop`; milliseconds between the two events, negative on error. */
+SPMM_EXPORT float SpMM_EventElapsedMs(void* start, void* stop);
+
+/*
  * File-to-file encoder used by model converters.  Stands in for
  *   extern "C" void GenSparseMatrixBinFile(char* DenseMatrixFileName, int M, int K,
  *                                          char* NZWeightsFileName, char* TileOffsetsFileName,
