@@ -67,6 +67,19 @@ extern "C" int SpMM_SplitK_API_Events(void* stream, const void* A, const void* C
                        KernelEnd);
 }
 
+extern "C" int SpMM_SplitK_Partials(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
+                                    void* Partials, int M, int N, int K, int Split_K)
+{
+    if (N != 8 && N != 16 && N != 32 && N != 64)
+        return tcsl_error_unknown();
+    if (M <= 0 || K <= 0 || M % tcsl::kTileRows != 0 || K % tcsl::kTileCols != 0 || Split_K < 1 ||
+        static_cast<long>(M / tcsl::kTileRows) * Split_K > 0x7fffffffL)
+        return tcsl_error_invalid_value();
+    if (!Compressed_A || !TileOffsets || !B || !Partials)
+        return tcsl_error_invalid_value();
+    return tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, Partials, M, N, K, Split_K);
+}
+
 extern "C" void* SpMM_EventCreate(void)
 {
     return tcsl_event_create();
@@ -127,21 +140,33 @@ int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, 
 
 extern "C" int SpMM_SuggestSplitK(int M, int N, int K)
 {
-    (void)N;
-    if (M <= 0 || K <= 0)
+    if (M <= 0 || K <= 0 || N <= 0)
         return 1;
-    // One wave per (128-row tile row, batch); a compute unit holds up to ten of
-    // them (LDS bound), and seven to eight per unit keep enough loads in flight.
+    // One wave per (128-row tile row, batch), spread over 256 compute units.  The stream a
+    // compute unit has to pull is the sum of its waves' tiles, and it needs about seven
+    // resident waves to pull at full rate, so the estimate to minimise is
+    //   max(ceil(units / 256), 7) * tiles_per_unit    busiest unit's share of the weight stream
+    // + units / 256 * slab_cost                       partial sums written, then read by the reduction
+    // in units of one 80 %-sparse tile (about 6.5 KB); ties go to the smaller split.
     const long row_tiles = (M + tcsl::kTileRows - 1) / tcsl::kTileRows;
     const long nkb = K / tcsl::kTileCols > 0 ? K / tcsl::kTileCols : 1;
-    const long target_waves = 256L * 8;
-    long s = (target_waves + row_tiles - 1) / row_tiles;
-    const long max_split = nkb / 4 > 0 ? nkb / 4 : 1;  // at least four tiles per batch
-    if (s > max_split)
-        s = max_split;
-    if (s < 1)
-        s = 1;
-    return static_cast<int>(s);
+    const double slab_cost = 2.0 * tcsl::kTileRows * N * 2.0 / 6554.0;
+    int best = 1;
+    double best_cost = 0.0;
+    for (long s = 1; s <= 32 && s <= nkb; s++) {
+        const long tiles = (nkb + s - 1) / s;
+        if (s > 1 && (tiles < 2 || tiles * (s - 1) >= nkb))
+            continue;  // batches of one tile, or a split that leaves the last batch empty
+        const long units = row_tiles * s;
+        const long waves_per_cu = (units + 255) / 256;
+        const double cost = static_cast<double>(waves_per_cu > 7 ? waves_per_cu : 7) * tiles +
+                            (s > 1 ? units / 256.0 * slab_cost : 0.0);
+        if (s == 1 || cost < best_cost - 1e-9) {
+            best = static_cast<int>(s);
+            best_cost = cost;
+        }
+    }
+    return best;
 }
 
 extern "C" void SpMM_SynthWeights(uint16_t* A_h, int M, int K, double sparsity, int row_skewed, uint64_t seed)

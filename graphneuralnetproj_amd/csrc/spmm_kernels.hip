@@ -8,22 +8,39 @@
 //
 // Design: "load as sparse, compute as dense", one wavefront per work unit.
 //   * A work unit is one 128-row tile row of A times one split-K batch of
-//     64-column tiles.  A workgroup is a single wave64, so no workgroup
-//     barrier exists anywhere: LDS operations of one wave execute in issue
-//     order, which is all the zero-fill -> scatter -> read-back chain needs.
-//   * Per 128x64 tile the wave streams the tile's packed (value,index) words
-//     from HBM with 128-bit buffer loads into registers (one tile ahead of
-//     use), clears a private 16 KiB LDS tile, scatters the fp16 values with
-//     ds_write_b16 at byte address 2*index (the index already carries the
-//     XOR swizzle that makes the read-back conflict free), reads the dense
-//     tile back as MFMA operands with ds_read_b128 and issues
-//     v_mfma_f32_16x16x32_f16 against the activation fragments, which come
-//     straight from global memory (they are L2 resident).
+//     64-column tiles.  A workgroup is a single wave64, so there is no
+//     workgroup barrier anywhere: LDS operations of one wave execute in issue
+//     order, which is all the scatter -> read-back -> clear chain needs.
+//   * The packed (value,index) words of a tile are streamed from HBM with
+//     non-temporal 128-bit buffer loads into a ring of register slots, a full
+//     tile ahead of their use.  The loads are inline assembly and their
+//     completion is awaited with hand-placed s_waitcnt vmcnt(N): every issue
+//     puts a fixed number of loads in flight, so N is a compile-time constant
+//     and the loads of the next tile stay in flight while this one is consumed.
+//   * A private 16 KiB LDS tile holds the dense 128x64 fp16 image.  It is
+//     cleared once; per tile the wave scatters the values with ds_write_b16 at
+//     byte address 2*index (the index already carries the XOR swizzle that makes
+//     the read-back conflict free), reads the tile back as MFMA operands with
+//     ds_read_b128, issues v_mfma_f32_16x16x32_f16 against activation fragments
+//     fetched straight from global memory (L2 resident), and then restores the
+//     zeros by writing 0 to the same addresses.  On gfx950 an LDS write costs
+//     about the same whatever its width, so undoing ~26 scatter instructions is
+//     cheaper than re-clearing 16 KiB.
+//   * TileOffsets of the unit sit in one VGPR (lane i = offset i) and are read
+//     with v_readlane, so the steady-state loop performs no scalar memory reads.
 //   * fp32 accumulators stay in registers over the whole batch; the epilogue
 //     rounds to fp16 and stores one slab of partial sums (or C itself when
 //     Split_K == 1).
+//
+// Rule for the asynchronous loads: the compiler does not know that the outputs of
+// the load asm statements arrive later.  A slot's registers may therefore only
+// become dead after a wait that covers the slot's loads -- consume() performs such
+// a wait on every path -- otherwise the register allocator could hand a register
+// with a load still in flight to an address computation.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <utility>
 
 namespace {
 
@@ -31,77 +48,133 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef u32x4 __attribute__((may_alias)) u32x4_a;
-typedef uint16_t __attribute__((may_alias)) u16_a;
+typedef int i32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kTileRows = 128;                      // rows of one encoded tile
-constexpr int kTileCols = 64;                       // columns of one encoded tile
+constexpr int kTileRows = 128;  // rows of one encoded tile
+constexpr int kTileCols = 64;   // columns of one encoded tile
 constexpr int kTileBytes = kTileRows * kTileCols * 2;
 constexpr int kWave = 64;
+constexpr int kVecPerLane = 8;  // 16-byte vectors per lane and ring slot: 512 vectors, i.e. tiles up to 25 % dense in one go
+constexpr int kRing = 2;        // ring slots: one tile being consumed, one in flight
 
-// Packed words of one tile, register resident: VPL 16-byte vectors per lane.
-template<int VPL>
-struct TileRegs {
-    u32x4 v[VPL];
-};
-
-// Issue the loads of one segment: up to VPL*64 consecutive vectors of one tile,
-// starting `rel` vectors into the unit's slice, of which `n` (> 0) belong to the
-// tile.  Always exactly VPL loads per lane, whatever n is, so that the
-// compiler's vmcnt bookkeeping is exact and the loads of the following segment
-// can stay in flight while this one is consumed.  Lanes past the end re-read the
-// last vector (scattering it twice is idempotent, and it is only scattered for
-// chunks that hold at least one real vector).  With the null descriptor nothing
-// is fetched at all.
-template<int VPL>
-__device__ __forceinline__ void load_segment(TileRegs<VPL>& r, __amdgpu_buffer_rsrc_t rsrc, int rel, int n, int lane)
+template<int... Is, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F&& f)
 {
-    const int last = rel + (n > 0 ? n - 1 : 0);
-#pragma unroll
-    for (int u = 0; u < VPL; u++) {
-        int v = rel + u * kWave + lane;
-        v = v < last ? v : last;
-        r.v[u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, v * 16, 0, 0);
-    }
+    (f(std::integral_constant<int, Is>{}), ...);
+}
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), fully unrolled
+template<int N, typename F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
 }
 
-__device__ __forceinline__ void scatter_vec(uint8_t* tile, u32x4 w)
+// 16 bytes per lane through a buffer descriptor; lanes at or past the descriptor's
+// size read zero and cause no memory traffic.  Non-temporal: the stream is read once.
+template<int IMM>
+__device__ __forceinline__ u32x4 load_words(i32x4 rsrc, int voff)
 {
-    // word = fp16 value | index << 16; byte address in the tile = 2 * index.
-    // The mask keeps a corrupt index inside the tile.
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-        uint32_t it = w[e];
-        *reinterpret_cast<u16_a*>(tile + ((it >> 15) & (kTileBytes - 2))) = static_cast<uint16_t>(it);
-    }
+    u32x4 r;
+    asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen offset:%3 nt" : "=v"(r) : "v"(voff), "s"(rsrc), "n"(IMM));
+    return r;
 }
 
-// One work unit.  NB = number of 16-token column blocks (N = 8 uses one block
-// with the upper 8 tokens masked to zero).
-template<int NB, int VPL>
+__device__ __forceinline__ half8 load_activations(const _Float16* p)
+{
+    half8 r;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r) : "v"(p));
+    return r;
+}
+
+// Wait until at most N vector-memory loads are outstanding (they complete in order).
+template<int N>
+__device__ __forceinline__ void wait_loads()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N < 63 ? N : 63));
+}
+
+// Ties a register to the preceding wait: later uses cannot be scheduled above it.
+template<typename T>
+__device__ __forceinline__ void settle(T& x)
+{
+    asm volatile("" : "+v"(x));
+}
+
+// Four packed words -> four 16-bit LDS writes of the value (or of zero) at byte
+// address 2 * (word >> 16).  One SDWA shift forms each address; all four are formed
+// first so the writes issue back to back.  Addresses are absolute LDS addresses: the
+// tile is the kernel's only LDS object and sits at address 0 (checked at entry).
+#define TCSL_ADDR(d, s) \
+    "v_lshlrev_b32_sdwa " d ", 1, " s " dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1\n"
+template<bool CLEAR>
+__device__ __forceinline__ void scatter_words(u32x4 w, uint32_t zero)
+{
+    uint32_t a0, a1, a2, a3;
+    if (!CLEAR)
+        asm volatile(TCSL_ADDR("%0", "%4") TCSL_ADDR("%1", "%5") TCSL_ADDR("%2", "%6") TCSL_ADDR("%3", "%7")
+                     "ds_write_b16 %0, %4\n ds_write_b16 %1, %5\n ds_write_b16 %2, %6\n ds_write_b16 %3, %7\n"
+                     : "=&v"(a0), "=&v"(a1), "=&v"(a2), "=&v"(a3)
+                     : "v"(w.x), "v"(w.y), "v"(w.z), "v"(w.w)
+                     : "memory");
+    else
+        asm volatile(TCSL_ADDR("%0", "%4") TCSL_ADDR("%1", "%5") TCSL_ADDR("%2", "%6") TCSL_ADDR("%3", "%7")
+                     "ds_write_b16 %0, %8\n ds_write_b16 %1, %8\n ds_write_b16 %2, %8\n ds_write_b16 %3, %8\n"
+                     : "=&v"(a0), "=&v"(a1), "=&v"(a2), "=&v"(a3)
+                     : "v"(w.x), "v"(w.y), "v"(w.z), "v"(w.w), "v"(zero)
+                     : "memory");
+}
+#undef TCSL_ADDR
+
+__device__ __forceinline__ void clear_tile(uint8_t* tile, int lane)
+{
+    typedef uint64_t __attribute__((may_alias)) u64_a;
+#pragma unroll
+    for (int u = 0; u < kTileBytes / (kWave * 8); u++)
+        *reinterpret_cast<u64_a*>(tile + u * (kWave * 8) + lane * 8) = 0;
+}
+
+// One work unit.  NB = number of 16-token column blocks; HALF = N is 8 (the upper
+// eight columns of the single block are computed on duplicates and dropped).
+template<int NB, bool HALF>
 __global__ __launch_bounds__(kWave) void tcsl_spmm_kernel(const u32x4* __restrict__ items,
                                                          const int* __restrict__ offsets,
                                                          const _Float16* __restrict__ B, _Float16* __restrict__ out,
                                                          int M, int N, int K, int split_k)
 {
     __shared__ __attribute__((aligned(16))) uint8_t tile[kTileBytes];
+    constexpr int VPL = kVecPerLane;
+    constexpr int D = kRing;
+    constexpr int L = VPL + 2 * NB;     // loads per issue: VPL word loads + 2 activation loads per column block
+    constexpr int kSeg = VPL * kWave;   // vectors per segment
+    if (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(tile)) != 0u)
+        return;  // scatter_words() assumes the tile starts at LDS address 0
 
     const int lane = threadIdx.x;
     const int row_tiles = M / kTileRows;
     const int rt = blockIdx.x % row_tiles;
     const int batch = blockIdx.x / row_tiles;
+    // split-K bookkeeping of the reference (csrc/SpMM_Kernel.cuh:312-320), clamped to the matrix
     const int nkb = K / kTileCols;
     const int avg = (nkb - 1) / split_k + 1;
     int kb0 = batch * avg;
     kb0 = kb0 < nkb ? kb0 : nkb;
     int kb1 = kb0 + avg;
     kb1 = kb1 < nkb ? kb1 : nkb;
+    const int ntile = kb1 - kb0;                          // tiles of this unit
+    const int* toff = offsets + (size_t)rt * nkb + kb0;   // toff[i] = first vector of tile i, toff[ntile] = end
 
-    const int* toff = offsets + (size_t)rt * nkb;  // offsets of this tile row, in vectors
-    const int unit_begin = toff[kb0];
-    const int unit_end = toff[kb1];
-    // Buffer descriptors cover this unit's slice only (see issue()): offsets stay
-    // below 4 GiB whatever the matrix size, and reads past the slice return zero.
+    // Offsets window: lane l holds toff[wbase + l].
+    int wbase = 0;
+    int wreg = toff[lane <= ntile ? lane : ntile];
+    auto tile_range = [&](int i, int& begin, int& end) {  // 0 <= i < ntile
+        if (i + 1 - wbase >= kWave) {  // slide the window (units longer than 63 tiles only)
+            wbase = i;
+            const int idx = i + lane;
+            wreg = toff[idx <= ntile ? idx : ntile];
+        }
+        begin = __builtin_amdgcn_readlane(wreg, i - wbase);
+        end = __builtin_amdgcn_readlane(wreg, i + 1 - wbase);
+    };
 
     f32x4 acc[NB][8];
 #pragma unroll
@@ -110,115 +183,182 @@ __global__ __launch_bounds__(kWave) void tcsl_spmm_kernel(const u32x4* __restric
         for (int r = 0; r < 8; r++)
             acc[c][r] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // MFMA operand geometry (v_mfma_f32_16x16x32_f16): lane l supplies row
-    // (l & 15) of the weight block and column (l & 15) of the activation
-    // block, both for the eight k values 8*(l >> 4) .. +7 of the 32-wide step.
+    // MFMA operand geometry (v_mfma_f32_16x16x32_f16): lane l supplies row (l & 15) of a
+    // 16-row weight block and column (l & 15) of a 16-token activation block, both for the
+    // eight k values 8*(l >> 4) .. +7 of the 32-wide step.
     const int l15 = lane & 15, q = lane >> 4;
-    // LDS byte offset of this lane's 16-byte granule for k-step s in row block 0;
-    // row blocks are 16 rows * 128 B = 2048 B apart.  Granule g of row r sits at
-    // position g ^ (r & 7) (the encoder's swizzle), and (r & 7) == (lane & 7).
+    // LDS byte offset of this lane's 16-byte granule for k-step s in row block 0; row blocks
+    // are 16 rows * 128 B apart.  Granule g of row r sits at position g ^ (r & 7) (the
+    // encoder's swizzle, csrc/SpMM_API.cu:330-339), and (r & 7) == (lane & 7).
     int a_off[2];
 #pragma unroll
     for (int s = 0; s < 2; s++)
         a_off[s] = l15 * 128 + (((s * 4 + q) ^ (lane & 7)) << 4);
 
-    // Activation fragment pointers: token-major B, one contiguous K vector per token.
+    // Activations: one contiguous K vector per token.
     const _Float16* bptr[NB];
-    bool btok[NB];
 #pragma unroll
     for (int c = 0; c < NB; c++) {
         int tok = c * 16 + l15;
-        btok[c] = tok < N;
-        bptr[c] = B + (size_t)(btok[c] ? tok : 0) * K + q * 8;
+        if (HALF)
+            tok &= 7;
+        bptr[c] = B + (size_t)tok * K + (size_t)kb0 * kTileCols + q * 8;
     }
+    // Per-lane byte offsets of the word loads: chunk u sits at lane*16 + u*1024 and the
+    // instruction's immediate offset reaches 4095.
+    const int voff_lo = lane * 16, voff_hi = lane * 16 + 4096;
+    uint32_t vzero = 0;
+    asm volatile("" : "+v"(vzero));  // a zero that stays in a VGPR for the clearing writes
 
-    // The stream of this unit is cut into segments: a tile of n vectors is
-    // ceil(n / (VPL*64)) segments (an empty tile is one empty segment).  The
-    // first segment of a tile clears the LDS tile, the last one multiplies.
-    constexpr int kSeg = VPL * kWave;
-    struct Cursor {
-        int kb;   // 64-column tile index within the tile row
-        int off;  // vectors of this tile covered by earlier segments
+    // The unit's stream is cut into segments of up to kSeg vectors that never cross a tile:
+    // a tile of n vectors is ceil(n / kSeg) segments, an empty tile one empty segment.
+    struct Seg {
+        int tile;     // index within the unit; ntile = past the end
+        int begin;    // first vector, absolute
+        int n;        // vectors in this segment
+        bool first;   // first segment of its tile
+        bool last;    // last segment of its tile
     };
-    auto next = [&](Cursor c) {
-        const int n = c.kb < kb1 ? toff[c.kb + 1] - toff[c.kb] : 0;
-        return (c.off + kSeg >= n) ? Cursor{c.kb + 1, 0} : Cursor{c.kb, c.off + kSeg};
+    struct Cur {
+        int tile, off;
+    };
+    auto make_seg = [&](Cur c, Seg& s, Cur& nxt) {
+        if (c.tile >= ntile) {
+            s = Seg{ntile, 0, 0, true, true};
+            nxt = c;
+            return;
+        }
+        int b, e;
+        tile_range(c.tile, b, e);
+        const int rest = e - b - c.off;
+        s.tile = c.tile;
+        s.begin = b + c.off;
+        s.n = rest < kSeg ? rest : kSeg;
+        s.first = c.off == 0;
+        s.last = rest <= kSeg;
+        nxt = s.last ? Cur{c.tile + 1, 0} : Cur{c.tile, c.off + kSeg};
     };
 
-    TileRegs<VPL> regs[2];
-    half8 bfrag[2][NB][2];
+    u32x4 regs[D][VPL];
+    half8 bfrag[D][NB][2];
+    Seg held[D];
 
-    // Loads are issued unconditionally (a cursor past the end reads through a
-    // null descriptor and a clamped activation pointer), again to keep the
-    // number of outstanding loads static.
-    auto issue = [&](int slot, Cursor c) {
-        const bool live = c.kb < kb1;
-        const int kb = live ? c.kb : kb1 - 1;
-        const int n = toff[kb + 1] - toff[kb] - c.off;
-        __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<u32x4*>(items + unit_begin), 0, live ? (unit_end - unit_begin) * 16 : 0, 0x00020000);
-        load_segment<VPL>(regs[slot], rs, toff[kb] - unit_begin + c.off, n < kSeg ? n : kSeg, lane);
+    // Always exactly L loads, whatever the segment holds, so the wait counts are static.
+    auto issue = [&](int slot, const Seg& s) {
+        const bool live = s.tile < ntile;
+        const uint64_t base = reinterpret_cast<uint64_t>(items + s.begin);
+        // descriptor over exactly this segment (nothing at all past the end of the unit)
+        i32x4 rs = {(int)(uint32_t)base, (int)((uint32_t)(base >> 32) & 0xffff), live ? s.n * 16 : 0, 0x00020000};
+        static_for<VPL>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            if constexpr (u < 4)
+                regs[slot][u] = load_words<u * 1024>(rs, voff_lo);
+            else
+                regs[slot][u] = load_words<(u - 4) * 1024>(rs, voff_hi);
+        });
+        const int bt = live ? s.tile : ntile - 1;
 #pragma unroll
         for (int cb = 0; cb < NB; cb++)
 #pragma unroll
-            for (int s = 0; s < 2; s++)
-                bfrag[slot][cb][s] = *reinterpret_cast<const half8*>(bptr[cb] + kb * kTileCols + s * 32);
+            for (int k = 0; k < 2; k++)
+                bfrag[slot][cb][k] = load_activations(bptr[cb] + bt * kTileCols + k * 32);
     };
 
-    auto consume = [&](int slot, Cursor c) {
-        const int n = toff[c.kb + 1] - toff[c.kb];
-        const int here = n - c.off;  // vectors from this segment's start to the tile's end
-        if (c.off == 0 && n > 0) {
-#pragma unroll
-            for (int u = 0; u < kTileBytes / (kWave * 16); u++)
-                *reinterpret_cast<u32x4_a*>(tile + u * (kWave * 16) + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+    // Y = loads issued after this slot's that may stay in flight.
+    auto consume = [&](int slot, const Seg& s, auto younger) {
+        constexpr int Y = decltype(younger)::value;
+        if (s.n == 0) {  // empty tile or past the end: only let the slot's loads land
+            wait_loads<Y>();
+            return;
         }
-#pragma unroll
-        for (int u = 0; u < VPL; u++)
-            if (u * kWave < here)
-                scatter_vec(tile, regs[slot].v[u]);
-        // the last segment of a non-empty tile: read back as dense operands and multiply
-        if (n > 0 && here <= kSeg) {
-#pragma unroll
-            for (int s = 0; s < 2; s++) {
-#pragma unroll
-                for (int r = 0; r < 8; r++) {
-                    half8 a = *reinterpret_cast<const half8*>(tile + a_off[s] + r * 2048);
-#pragma unroll
-                    for (int cb = 0; cb < NB; cb++) {
-                        half8 bv = bfrag[slot][cb][s];
-                        if (!btok[cb])
-                            bv = half8{0, 0, 0, 0, 0, 0, 0, 0};
-                        acc[cb][r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bv, acc[cb][r], 0, 0, 0);
-                    }
-                }
+        static_for<VPL>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            if (u * kWave < s.n) {
+                wait_loads<Y + (L - 1 - u)>();
+                settle(regs[slot][u]);
+                if ((u + 1) * kWave <= s.n)
+                    scatter_words<false>(regs[slot][u], vzero);
+                else if (u * kWave + lane < s.n)  // the segment's last, partial chunk
+                    scatter_words<false>(regs[slot][u], vzero);
             }
+        });
+        wait_loads<Y>();
+        if (!s.last)
+            return;  // more segments of this tile follow
+#pragma unroll
+        for (int cb = 0; cb < NB; cb++)
+#pragma unroll
+            for (int k = 0; k < 2; k++)
+                settle(bfrag[slot][cb][k]);
+        // read the dense tile back and multiply; all reads of a pass are issued before its MFMAs
+        constexpr int kPasses = NB == 1 ? 1 : 2;
+        constexpr int kStepsPerPass = 2 / kPasses;
+#pragma unroll
+        for (int p = 0; p < kPasses; p++) {
+            half8 afrag[kStepsPerPass][8];
+#pragma unroll
+            for (int k = 0; k < kStepsPerPass; k++)
+#pragma unroll
+                for (int r = 0; r < 8; r++)
+                    afrag[k][r] = *reinterpret_cast<const half8*>(tile + a_off[p * kStepsPerPass + k] + r * 2048);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int k = 0; k < kStepsPerPass; k++)
+#pragma unroll
+                for (int r = 0; r < 8; r++)
+#pragma unroll
+                    for (int cb = 0; cb < NB; cb++)
+                        acc[cb][r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                            afrag[k][r], bfrag[slot][cb][p * kStepsPerPass + k], acc[cb][r], 0, 0, 0);
+        }
+        // restore the all-zero tile: undo this segment's writes, or clear everything when
+        // earlier segments (whose words are gone) wrote into it as well
+        if (!s.first) {
+            clear_tile(tile, lane);
+        } else {
+            static_for<VPL>([&](auto uc) {
+                constexpr int u = decltype(uc)::value;
+                if (u * kWave < s.n) {
+                    if ((u + 1) * kWave <= s.n)
+                        scatter_words<true>(regs[slot][u], vzero);
+                    else if (u * kWave + lane < s.n)
+                        scatter_words<true>(regs[slot][u], vzero);
+                }
+            });
         }
     };
 
-    if (kb0 < kb1) {
-        Cursor c0{kb0, 0};
-        issue(0, c0);
-        for (;;) {
-            Cursor c1 = next(c0);
-            issue(1, c1);
-            consume(0, c0);
-            if (c1.kb >= kb1)
-                break;
-            c0 = next(c1);
-            issue(0, c0);
-            consume(1, c1);
-            if (c0.kb >= kb1)
-                break;
+    if (ntile > 0) {
+        clear_tile(tile, lane);
+        Cur ci{0, 0};
+#pragma unroll
+        for (int s = 0; s < D; s++) {
+            Cur nx;
+            make_seg(ci, held[s], nx);
+            ci = nx;
+            issue(s, held[s]);
         }
+        for (;;) {
+#pragma unroll
+            for (int s = 0; s < D; s++) {
+                consume(s, held[s], std::integral_constant<int, (D - 1) * L>{});
+                Cur nx;
+                make_seg(ci, held[s], nx);
+                ci = nx;
+                issue(s, held[s]);
+            }
+            if (held[0].tile >= ntile)
+                break;  // every later slot is past the end as well
+        }
+        wait_loads<0>();
     }
 
-    // Epilogue.  acc[c][r][i] is output row r*16 + 4*q + i of this tile row for
-    // token c*16 + l15; the output keeps one contiguous M vector per token.
+    // Epilogue.  acc[c][r][i] is output row r*16 + 4*q + i of this tile row for token
+    // c*16 + l15; the output keeps one contiguous M vector per token.
     _Float16* obase = out + (size_t)batch * M * N + (size_t)rt * kTileRows + q * 4;
 #pragma unroll
     for (int c = 0; c < NB; c++) {
-        if (!btok[c])
+        if (HALF && l15 >= 8)
             continue;
         _Float16* o = obase + (size_t)(c * 16 + l15) * M;
 #pragma unroll
@@ -260,12 +400,12 @@ __global__ __launch_bounds__(256) void tcsl_copy_kernel(u32x4* __restrict__ dst,
         dst[i] = src[i];
 }
 
-template<int NB, int VPL>
+template<int NB, bool HALF>
 int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const void* B, void* out, int M, int N,
                 int K, int split_k)
 {
     const int units = (M / kTileRows) * split_k;
-    hipLaunchKernelGGL((tcsl_spmm_kernel<NB, VPL>), dim3(units), dim3(kWave), 0, stream,
+    hipLaunchKernelGGL((tcsl_spmm_kernel<NB, HALF>), dim3(units), dim3(kWave), 0, stream,
                        static_cast<const u32x4*>(items), offsets, static_cast<const _Float16*>(B),
                        static_cast<_Float16*>(out), M, N, K, split_k);
     return static_cast<int>(hipGetLastError());
@@ -283,12 +423,13 @@ extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offs
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (N) {
         case 8:
+            return launch_spmm<1, true>(s, items, offsets, B, out, M, N, K, split_k);
         case 16:
-            return launch_spmm<1, 8>(s, items, offsets, B, out, M, N, K, split_k);
+            return launch_spmm<1, false>(s, items, offsets, B, out, M, N, K, split_k);
         case 32:
-            return launch_spmm<2, 8>(s, items, offsets, B, out, M, N, K, split_k);
+            return launch_spmm<2, false>(s, items, offsets, B, out, M, N, K, split_k);
         case 64:
-            return launch_spmm<4, 8>(s, items, offsets, B, out, M, N, K, split_k);
+            return launch_spmm<4, false>(s, items, offsets, B, out, M, N, K, split_k);
         default:
             return static_cast<int>(hipErrorInvalidValue);
     }

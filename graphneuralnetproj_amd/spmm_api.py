@@ -34,6 +34,7 @@ EXPORTED_SYMBOLS = (
     "SpMM_SynthActivations",
     "SpMM_CalibrationCopy",
     "SpMM_SplitK_API_Events",
+    "SpMM_SplitK_Partials",
     "SpMM_EventCreate",
     "SpMM_EventDestroy",
     "SpMM_EventRecord",
@@ -105,6 +106,8 @@ def load_library():
     lib.SpMM_CalibrationCopy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_long]
     lib.SpMM_SplitK_API_Events.restype = ctypes.c_int
     lib.SpMM_SplitK_API_Events.argtypes = lib.SpMM_SplitK_API.argtypes + [ctypes.c_void_p, ctypes.c_void_p]
+    lib.SpMM_SplitK_Partials.restype = ctypes.c_int
+    lib.SpMM_SplitK_Partials.argtypes = [ctypes.c_void_p] * 5 + [ctypes.c_int] * 4
     lib.SpMM_EventCreate.restype = ctypes.c_void_p
     lib.SpMM_EventCreate.argtypes = []
     lib.SpMM_EventDestroy.restype = None

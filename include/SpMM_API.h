@@ -85,6 +85,16 @@ SPMM_EXPORT int SpMM_SplitK_API(void* stream, const void* A, const void* Compres
 SPMM_EXPORT int SpMM_SplitK_API_Events(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets,
                                        const void* B, void* C, int M_Global, int N_Global, int K_Global,
                                        void* Reduction_Workspace, int Split_K, void* KernelBegin, void* KernelEnd);
+/*
+ * The first half of SpMM_SplitK_API alone: batch b's fp16 partial sums go to
+ * Partials[b*M*N ..) (Split_K*M*N values; with Split_K == 1 that is the product itself)
+ * and no reduction follows.  Lets a caller fuse its own reduction, and lets a benchmark
+ * time the main kernel back to back.  Same checks and return codes as SpMM_SplitK_API
+ * (nothing is printed).  The reference has no such entry point; its kernel writes the
+ * same slabs (csrc/SpMM_Kernel.cuh:731-734).
+ */
+SPMM_EXPORT int SpMM_SplitK_Partials(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
+                                     void* Partials, int M_Global, int N_Global, int K_Global, int Split_K);
 SPMM_EXPORT void* SpMM_EventCreate(void);
 SPMM_EXPORT void SpMM_EventDestroy(void* event);
 SPMM_EXPORT int SpMM_EventRecord(void* event, void* stream);
