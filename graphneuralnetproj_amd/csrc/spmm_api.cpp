@@ -10,7 +10,7 @@
 
 extern "C" {
 int tcsl_launch_spmm(void* stream, const void* items, const int* offsets, const void* B, void* out, int M, int N,
-                     int K, int split_k);
+                     int K, int split_k, int waves, int stage_b, unsigned lds_bytes);
 int tcsl_launch_reduce(void* stream, void* C, const void* W, long mn, int split_k);
 int tcsl_launch_copy(void* stream, void* dst, const void* src, long bytes);
 void* tcsl_event_create(void);
@@ -46,6 +46,60 @@ extern "C" const char* SpMM_GetErrorString(int code)
 }
 
 namespace {
+
+// Launch shape of the main kernel: W waves per workgroup (each wave owns one 128-row tile
+// row of one batch), and whether the batch's activation slice is staged in LDS.
+struct LaunchPlan {
+    int waves;
+    int stage_b;
+    unsigned lds_bytes;
+};
+
+LaunchPlan plan_launch(int M, int N, int K, int Split_K)
+{
+    constexpr long kLds = 160 * 1024, kTile = 16384, kCUs = 256;
+    const long row_tiles = M / tcsl::kTileRows;
+    const long nkb = K / tcsl::kTileCols;
+    const long tiles = (nkb - 1) / Split_K + 1;  // tiles of the longest batch
+    if (N > 16)  // wide accumulators: one wave per workgroup, activations from global memory
+        return LaunchPlan{1, 0, static_cast<unsigned>(kTile)};
+    const long slice = tiles * (N == 8 ? 8 : 16) * 128;  // staged activation bytes
+    // Pick W: the busiest compute unit runs ceil(workgroups / 256) workgroups of W waves of
+    // `tiles` tiles each, and pulls its stream at full rate only with about seven waves
+    // resident.  Ties go to the larger W (more waves share one staged slice).
+    LaunchPlan best{1, 0, static_cast<unsigned>(kTile)};
+    double best_cost = 0.0;
+    for (int w = 1; w <= 8; w++) {
+        for (int stage = 0; stage <= 1; stage++) {
+            const long lds = w * kTile + (stage ? slice : 0);
+            if (lds > kLds)
+                continue;
+            const long wgs = (row_tiles + w - 1) / w * Split_K;
+            long fit = kLds / lds;  // workgroups resident per compute unit
+            if (fit > 8 / w)
+                fit = 8 / w;        // eight waves per compute unit at this kernel's register use
+            const long per_cu = (wgs + kCUs - 1) / kCUs;
+            const long resident = (per_cu < fit ? per_cu : fit) * w;
+            double cost = static_cast<double>(per_cu) * w * tiles * (resident < 7 ? 7.0 / resident : 1.0);
+            if (!stage)
+                cost *= 1.03;  // activations re-fetched through L2 for every tile
+            if (best_cost == 0.0 || cost <= best_cost * (1.0 + 1e-9)) {
+                best = LaunchPlan{w, stage, static_cast<unsigned>(lds)};
+                best_cost = cost;
+            }
+        }
+    }
+    return best;
+}
+
+int launch_main(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* out, int M, int N,
+                int K, int Split_K)
+{
+    const LaunchPlan p = plan_launch(M, N, K, Split_K);
+    return tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, out, M, N, K, Split_K, p.waves, p.stage_b,
+                            p.lds_bytes);
+}
+
 int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* C, int M, int N,
                 int K, void* Reduction_Workspace, int Split_K, void* ev_begin, void* ev_end);
 }
@@ -77,7 +131,7 @@ extern "C" int SpMM_SplitK_Partials(void* stream, const void* Compressed_A, cons
         return tcsl_error_invalid_value();
     if (!Compressed_A || !TileOffsets || !B || !Partials)
         return tcsl_error_invalid_value();
-    return tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, Partials, M, N, K, Split_K);
+    return launch_main(stream, Compressed_A, TileOffsets, B, Partials, M, N, K, Split_K);
 }
 
 extern "C" void* SpMM_EventCreate(void)
@@ -101,6 +155,7 @@ extern "C" float SpMM_EventElapsedMs(void* start, void* stop)
 }
 
 namespace {
+
 int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* C, int M, int N,
                 int K, void* Reduction_Workspace, int Split_K, void* ev_begin, void* ev_end)
 {
@@ -126,8 +181,7 @@ int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, 
     int rc = 0;
     if (ev_begin && (rc = tcsl_event_record(ev_begin, stream)) != 0)
         return rc;
-    rc = tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, Split_K == 1 ? C : Reduction_Workspace, M, N, K,
-                          Split_K);
+    rc = launch_main(stream, Compressed_A, TileOffsets, B, Split_K == 1 ? C : Reduction_Workspace, M, N, K, Split_K);
     if (rc != 0)
         return rc;
     if (ev_end && (rc = tcsl_event_record(ev_end, stream)) != 0)

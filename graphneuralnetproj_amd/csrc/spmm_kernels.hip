@@ -8,9 +8,14 @@
 //
 // Design: "load as sparse, compute as dense", one wavefront per work unit.
 //   * A work unit is one 128-row tile row of A times one split-K batch of
-//     64-column tiles.  A workgroup is a single wave64, so there is no
-//     workgroup barrier anywhere: LDS operations of one wave execute in issue
-//     order, which is all the scatter -> read-back -> clear chain needs.
+//     64-column tiles, and one wave64 owns it from start to finish: LDS
+//     operations of one wave execute in issue order, which is all the
+//     scatter -> read-back -> clear chain needs, so the loop has no barrier.
+//   * A workgroup is W such waves on consecutive tile rows of the same batch.
+//     They share nothing but the batch's activation slice, staged once into LDS
+//     (one barrier, before the loop), and the fact that W units land on one
+//     compute unit: the host picks W so that the grid is one workgroup per
+//     compute unit where the shape allows it.
 //   * The packed (value,index) words of a tile are streamed from HBM with
 //     non-temporal 128-bit buffer loads into a ring of register slots, a full
 //     tile ahead of their use.  The loads are inline assembly and their
@@ -22,15 +27,17 @@
 //     byte address 2*index (the index already carries the XOR swizzle that makes
 //     the read-back conflict free), reads the tile back as MFMA operands with
 //     ds_read_b128, issues v_mfma_f32_16x16x32_f16 against activation fragments
-//     fetched straight from global memory (L2 resident), and then restores the
-//     zeros by writing 0 to the same addresses.  On gfx950 an LDS write costs
+//     read from the staged slice (or, when the slice does not fit, fetched
+//     straight from global memory, where they are L2 resident), and then restores
+//     the zeros by writing 0 to the same addresses.  On gfx950 an LDS write costs
 //     about the same whatever its width, so undoing ~26 scatter instructions is
 //     cheaper than re-clearing 16 KiB.
 //   * TileOffsets of the unit sit in one VGPR (lane i = offset i) and are read
 //     with v_readlane, so the steady-state loop performs no scalar memory reads.
 //   * fp32 accumulators stay in registers over the whole batch; the epilogue
-//     rounds to fp16 and stores one slab of partial sums (or C itself when
-//     Split_K == 1).
+//     rounds to fp16, transposes through the wave's (by then free) LDS tile and
+//     stores whole 256-byte token rows of one slab of partial sums (or of C
+//     itself when Split_K == 1).
 //
 // Rule for the asynchronous loads: the compiler does not know that the outputs of
 // the load asm statements arrive later.  A slot's registers may therefore only
@@ -40,6 +47,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <utility>
 
 namespace {
@@ -56,6 +64,7 @@ constexpr int kTileBytes = kTileRows * kTileCols * 2;
 constexpr int kWave = 64;
 constexpr int kVecPerLane = 8;  // 16-byte vectors per lane and ring slot: 512 vectors, i.e. tiles up to 25 % dense in one go
 constexpr int kRing = 2;        // ring slots: one tile being consumed, one in flight
+constexpr unsigned kMaxLdsBytes = 160 * 1024;  // LDS of one gfx950 compute unit
 
 template<int... Is, typename F>
 __device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F&& f)
@@ -101,26 +110,24 @@ __device__ __forceinline__ void settle(T& x)
 }
 
 // Four packed words -> four 16-bit LDS writes of the value (or of zero) at byte
-// address 2 * (word >> 16).  One SDWA shift forms each address; all four are formed
-// first so the writes issue back to back.  Addresses are absolute LDS addresses: the
-// tile is the kernel's only LDS object and sits at address 0 (checked at entry).
-#define TCSL_ADDR(d, s) \
-    "v_lshlrev_b32_sdwa " d ", 1, " s " dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1\n"
+// address base + 2 * (word >> 16).  One v_mad_u32_u16 on the word's high half forms
+// each address; all four are formed first so the writes issue back to back.
+#define TCSL_ADDR(d, s) "v_mad_u32_u16 " d ", " s ", %9, %8 op_sel:[1,0,0,0]\n"
 template<bool CLEAR>
-__device__ __forceinline__ void scatter_words(u32x4 w, uint32_t zero)
+__device__ __forceinline__ void scatter_words(u32x4 w, uint32_t base, uint32_t two, uint32_t zero)
 {
     uint32_t a0, a1, a2, a3;
     if (!CLEAR)
         asm volatile(TCSL_ADDR("%0", "%4") TCSL_ADDR("%1", "%5") TCSL_ADDR("%2", "%6") TCSL_ADDR("%3", "%7")
                      "ds_write_b16 %0, %4\n ds_write_b16 %1, %5\n ds_write_b16 %2, %6\n ds_write_b16 %3, %7\n"
                      : "=&v"(a0), "=&v"(a1), "=&v"(a2), "=&v"(a3)
-                     : "v"(w.x), "v"(w.y), "v"(w.z), "v"(w.w)
+                     : "v"(w.x), "v"(w.y), "v"(w.z), "v"(w.w), "v"(base), "v"(two)
                      : "memory");
     else
         asm volatile(TCSL_ADDR("%0", "%4") TCSL_ADDR("%1", "%5") TCSL_ADDR("%2", "%6") TCSL_ADDR("%3", "%7")
-                     "ds_write_b16 %0, %8\n ds_write_b16 %1, %8\n ds_write_b16 %2, %8\n ds_write_b16 %3, %8\n"
+                     "ds_write_b16 %0, %10\n ds_write_b16 %1, %10\n ds_write_b16 %2, %10\n ds_write_b16 %3, %10\n"
                      : "=&v"(a0), "=&v"(a1), "=&v"(a2), "=&v"(a3)
-                     : "v"(w.x), "v"(w.y), "v"(w.z), "v"(w.w), "v"(zero)
+                     : "v"(w.x), "v"(w.y), "v"(w.z), "v"(w.w), "v"(base), "v"(two), "v"(zero)
                      : "memory");
 }
 #undef TCSL_ADDR
@@ -133,26 +140,34 @@ __device__ __forceinline__ void clear_tile(uint8_t* tile, int lane)
         *reinterpret_cast<u64_a*>(tile + u * (kWave * 8) + lane * 8) = 0;
 }
 
-// One work unit.  NB = number of 16-token column blocks; HALF = N is 8 (the upper
-// eight columns of the single block are computed on duplicates and dropped).
-template<int NB, bool HALF>
-__global__ __launch_bounds__(kWave) void tcsl_spmm_kernel(const u32x4* __restrict__ items,
-                                                         const int* __restrict__ offsets,
-                                                         const _Float16* __restrict__ B, _Float16* __restrict__ out,
-                                                         int M, int N, int K, int split_k)
+// blockDim.x = W * 64.  Wave w of workgroup g owns tile row (g % groups) * W + w of batch
+// g / groups, groups = ceil(tile rows / W).  NB = number of 16-token column blocks;
+// HALF = N is 8 (the upper eight columns of the single block are computed on duplicates
+// and dropped); BLDS = the batch's activation slice is staged in LDS; MAXW bounds W and
+// with it the registers a wave may use.
+// Dynamic LDS: W tiles of 16 KiB, then (BLDS) tiles_per_batch * tokens * 128 bytes.
+template<int NB, bool HALF, bool BLDS, int MAXW>
+__global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __restrict__ items,
+                                                                const int* __restrict__ offsets,
+                                                                const _Float16* __restrict__ B,
+                                                                _Float16* __restrict__ out, int M, int N, int K,
+                                                                int split_k)
 {
-    __shared__ __attribute__((aligned(16))) uint8_t tile[kTileBytes];
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int VPL = kVecPerLane;
     constexpr int D = kRing;
-    constexpr int L = VPL + 2 * NB;     // loads per issue: VPL word loads + 2 activation loads per column block
-    constexpr int kSeg = VPL * kWave;   // vectors per segment
-    if (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(tile)) != 0u)
-        return;  // scatter_words() assumes the tile starts at LDS address 0
+    constexpr int L = VPL + (BLDS ? 0 : 2 * NB);  // loads per issue: word loads (+ activation loads)
+    constexpr int kSeg = VPL * kWave;             // vectors per segment
+    constexpr int NTOK = HALF ? 8 : NB * 16;      // tokens in the staged slice
 
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int W = blockDim.x / kWave;
     const int row_tiles = M / kTileRows;
-    const int rt = blockIdx.x % row_tiles;
-    const int batch = blockIdx.x / row_tiles;
+    const int groups = (row_tiles + W - 1) / W;
+    const int batch = blockIdx.x / groups;
+    const int rt = (blockIdx.x % groups) * W + wave;
+    const bool active = rt < row_tiles;
     // split-K bookkeeping of the reference (csrc/SpMM_Kernel.cuh:312-320), clamped to the matrix
     const int nkb = K / kTileCols;
     const int avg = (nkb - 1) / split_k + 1;
@@ -160,12 +175,31 @@ __global__ __launch_bounds__(kWave) void tcsl_spmm_kernel(const u32x4* __restric
     kb0 = kb0 < nkb ? kb0 : nkb;
     int kb1 = kb0 + avg;
     kb1 = kb1 < nkb ? kb1 : nkb;
-    const int ntile = kb1 - kb0;                          // tiles of this unit
-    const int* toff = offsets + (size_t)rt * nkb + kb0;   // toff[i] = first vector of tile i, toff[ntile] = end
+    const int ntile = kb1 - kb0;  // tiles of this unit
+    uint8_t* const tile = lds + wave * kTileBytes;
+    uint8_t* const bslice = lds + W * kTileBytes;  // [tile][token][8 granules of 16 B at position g ^ (token & 7)]
 
-    // Offsets window: lane l holds toff[wbase + l].
+    // Offsets window: lane l holds toff[wbase + l]; toff[i] = first vector of tile i,
+    // toff[ntile] = end.  Issued first so its latency overlaps the staging below.
+    const int* toff = offsets + (size_t)(active ? rt : 0) * nkb + kb0;
     int wbase = 0;
     int wreg = toff[lane <= ntile ? lane : ntile];
+
+    if (BLDS) {
+        const int ngran = ntile * NTOK * 8;
+        for (int id = threadIdx.x; id < ngran; id += blockDim.x) {
+            const int j = id / (NTOK * 8), t = (id >> 3) % NTOK, g = id & 7;
+            const half8 v = *reinterpret_cast<const half8*>(B + (size_t)t * K + (size_t)(kb0 + j) * kTileCols + g * 8);
+            *reinterpret_cast<half8*>(bslice + (size_t)j * (NTOK * 128) + t * 128 + ((g ^ (t & 7)) << 4)) = v;
+        }
+    }
+    if (active)
+        clear_tile(tile, lane);
+    if (BLDS)
+        __syncthreads();  // the only barrier: every wave of the workgroup reaches it
+    if (!active)
+        return;
+
     auto tile_range = [&](int i, int& begin, int& end) {  // 0 <= i < ntile
         if (i + 1 - wbase >= kWave) {  // slide the window (units longer than 63 tiles only)
             wbase = i;
@@ -195,20 +229,26 @@ __global__ __launch_bounds__(kWave) void tcsl_spmm_kernel(const u32x4* __restric
     for (int s = 0; s < 2; s++)
         a_off[s] = l15 * 128 + (((s * 4 + q) ^ (lane & 7)) << 4);
 
-    // Activations: one contiguous K vector per token.
+    // Activations: one contiguous K vector per token in global memory; in the staged
+    // slice the same granule swizzle as the weight tile keeps the reads conflict free.
     const _Float16* bptr[NB];
+    int b_off[NB][2];
 #pragma unroll
     for (int c = 0; c < NB; c++) {
         int tok = c * 16 + l15;
         if (HALF)
             tok &= 7;
         bptr[c] = B + (size_t)tok * K + (size_t)kb0 * kTileCols + q * 8;
+#pragma unroll
+        for (int s = 0; s < 2; s++)
+            b_off[c][s] = tok * 128 + (((s * 4 + q) ^ (tok & 7)) << 4);
     }
     // Per-lane byte offsets of the word loads: chunk u sits at lane*16 + u*1024 and the
     // instruction's immediate offset reaches 4095.
     const int voff_lo = lane * 16, voff_hi = lane * 16 + 4096;
-    uint32_t vzero = 0;
-    asm volatile("" : "+v"(vzero));  // a zero that stays in a VGPR for the clearing writes
+    // constants the scatter asm wants in VGPRs
+    uint32_t vzero = 0, vtwo = 2, vbase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(tile));
+    asm volatile("" : "+v"(vzero), "+v"(vtwo), "+v"(vbase));
 
     // The unit's stream is cut into segments of up to kSeg vectors that never cross a tile:
     // a tile of n vectors is ceil(n / kSeg) segments, an empty tile one empty segment.
@@ -240,7 +280,7 @@ __global__ __launch_bounds__(kWave) void tcsl_spmm_kernel(const u32x4* __restric
     };
 
     u32x4 regs[D][VPL];
-    half8 bfrag[D][NB][2];
+    half8 bfrag[D][NB][2];  // only used when the activations come from global memory
     Seg held[D];
 
     // Always exactly L loads, whatever the segment holds, so the wait counts are static.
@@ -256,12 +296,14 @@ __global__ __launch_bounds__(kWave) void tcsl_spmm_kernel(const u32x4* __restric
             else
                 regs[slot][u] = load_words<(u - 4) * 1024>(rs, voff_hi);
         });
-        const int bt = live ? s.tile : ntile - 1;
+        if (!BLDS) {
+            const int bt = live ? s.tile : ntile - 1;
 #pragma unroll
-        for (int cb = 0; cb < NB; cb++)
+            for (int cb = 0; cb < NB; cb++)
 #pragma unroll
-            for (int k = 0; k < 2; k++)
-                bfrag[slot][cb][k] = load_activations(bptr[cb] + bt * kTileCols + k * 32);
+                for (int k = 0; k < 2; k++)
+                    bfrag[slot][cb][k] = load_activations(bptr[cb] + bt * kTileCols + k * 32);
+        }
     };
 
     // Y = loads issued after this slot's that may stay in flight.
@@ -277,19 +319,31 @@ __global__ __launch_bounds__(kWave) void tcsl_spmm_kernel(const u32x4* __restric
                 wait_loads<Y + (L - 1 - u)>();
                 settle(regs[slot][u]);
                 if ((u + 1) * kWave <= s.n)
-                    scatter_words<false>(regs[slot][u], vzero);
+                    scatter_words<false>(regs[slot][u], vbase, vtwo, vzero);
                 else if (u * kWave + lane < s.n)  // the segment's last, partial chunk
-                    scatter_words<false>(regs[slot][u], vzero);
+                    scatter_words<false>(regs[slot][u], vbase, vtwo, vzero);
             }
         });
         wait_loads<Y>();
         if (!s.last)
             return;  // more segments of this tile follow
+        half8 bf[NB][2];
+        if (BLDS) {
+            const uint8_t* bt = bslice + (size_t)s.tile * (NTOK * 128);
 #pragma unroll
-        for (int cb = 0; cb < NB; cb++)
+            for (int cb = 0; cb < NB; cb++)
 #pragma unroll
-            for (int k = 0; k < 2; k++)
-                settle(bfrag[slot][cb][k]);
+                for (int k = 0; k < 2; k++)
+                    bf[cb][k] = *reinterpret_cast<const half8*>(bt + b_off[cb][k]);
+        } else {
+#pragma unroll
+            for (int cb = 0; cb < NB; cb++)
+#pragma unroll
+                for (int k = 0; k < 2; k++) {
+                    settle(bfrag[slot][cb][k]);
+                    bf[cb][k] = bfrag[slot][cb][k];
+                }
+        }
         // read the dense tile back and multiply; all reads of a pass are issued before its MFMAs
         constexpr int kPasses = NB == 1 ? 1 : 2;
         constexpr int kStepsPerPass = 2 / kPasses;
@@ -308,8 +362,8 @@ __global__ __launch_bounds__(kWave) void tcsl_spmm_kernel(const u32x4* __restric
                 for (int r = 0; r < 8; r++)
 #pragma unroll
                     for (int cb = 0; cb < NB; cb++)
-                        acc[cb][r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                            afrag[k][r], bfrag[slot][cb][p * kStepsPerPass + k], acc[cb][r], 0, 0, 0);
+                        acc[cb][r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[k][r], bf[cb][p * kStepsPerPass + k],
+                                                                            acc[cb][r], 0, 0, 0);
         }
         // restore the all-zero tile: undo this segment's writes, or clear everything when
         // earlier segments (whose words are gone) wrote into it as well
@@ -320,16 +374,15 @@ __global__ __launch_bounds__(kWave) void tcsl_spmm_kernel(const u32x4* __restric
                 constexpr int u = decltype(uc)::value;
                 if (u * kWave < s.n) {
                     if ((u + 1) * kWave <= s.n)
-                        scatter_words<true>(regs[slot][u], vzero);
+                        scatter_words<true>(regs[slot][u], vbase, vtwo, vzero);
                     else if (u * kWave + lane < s.n)
-                        scatter_words<true>(regs[slot][u], vzero);
+                        scatter_words<true>(regs[slot][u], vbase, vtwo, vzero);
                 }
             });
         }
     };
 
     if (ntile > 0) {
-        clear_tile(tile, lane);
         Cur ci{0, 0};
 #pragma unroll
         for (int s = 0; s < D; s++) {
@@ -354,20 +407,33 @@ __global__ __launch_bounds__(kWave) void tcsl_spmm_kernel(const u32x4* __restric
     }
 
     // Epilogue.  acc[c][r][i] is output row r*16 + 4*q + i of this tile row for token
-    // c*16 + l15; the output keeps one contiguous M vector per token.
-    _Float16* obase = out + (size_t)batch * M * N + (size_t)rt * kTileRows + q * 4;
+    // c*16 + l15; the output keeps one contiguous M vector per token.  The block goes through
+    // the wave's LDS tile as [token][128 rows] (token stride padded to 272 B) so that the
+    // global stores are 16 bytes per lane with 16 lanes covering a token's 256 bytes.
+    constexpr int kTokStride = 272;
+    constexpr int kTok = HALF ? 8 : 16;
+    _Float16* oslab = out + (size_t)batch * M * N + (size_t)rt * kTileRows;
 #pragma unroll
     for (int c = 0; c < NB; c++) {
-        if (HALF && l15 >= 8)
-            continue;
-        _Float16* o = obase + (size_t)(c * 16 + l15) * M;
+        // the clearing writes of the last tile (inline asm, unknown to the compiler's own
+        // LDS bookkeeping) and the previous block's reads must be done before the tile is reused
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (!(HALF && l15 >= 8)) {
 #pragma unroll
-        for (int r = 0; r < 8; r++) {
-            half4 h;
+            for (int r = 0; r < 8; r++) {
+                half4 h;
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-                h[i] = static_cast<_Float16>(acc[c][r][i]);
-            *reinterpret_cast<half4*>(o + r * 16) = h;
+                for (int i = 0; i < 4; i++)
+                    h[i] = static_cast<_Float16>(acc[c][r][i]);
+                *reinterpret_cast<half4*>(tile + l15 * kTokStride + (r * 16 + q * 4) * 2) = h;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kTok / 4; i++) {
+            const int e = i * kWave + lane;
+            const int tok = e >> 4, part = e & 15;
+            const half8 v = *reinterpret_cast<const half8*>(tile + tok * kTokStride + part * 16);
+            *reinterpret_cast<half8*>(oslab + (size_t)(c * 16 + tok) * M + part * 8) = v;
         }
     }
 }
@@ -400,12 +466,29 @@ __global__ __launch_bounds__(256) void tcsl_copy_kernel(u32x4* __restrict__ dst,
         dst[i] = src[i];
 }
 
-template<int NB, bool HALF>
+template<int NB, bool HALF, bool BLDS, int MAXW>
 int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const void* B, void* out, int M, int N,
-                int K, int split_k)
+                int K, int split_k, int waves, unsigned lds_bytes)
 {
-    const int units = (M / kTileRows) * split_k;
-    hipLaunchKernelGGL((tcsl_spmm_kernel<NB, HALF>), dim3(units), dim3(kWave), 0, stream,
+    if (waves < 1 || waves > MAXW || lds_bytes > kMaxLdsBytes)
+        return static_cast<int>(hipErrorInvalidValue);
+    auto kernel = tcsl_spmm_kernel<NB, HALF, BLDS, MAXW>;
+    // more than 64 KiB of dynamic LDS has to be allowed once per kernel (per device, re-armed lazily)
+    static std::atomic<int> armed_device{-1};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess)
+        return static_cast<int>(e);
+    if (armed_device.load(std::memory_order_acquire) != dev) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                kMaxLdsBytes);
+        if (e != hipSuccess)
+            return static_cast<int>(e);
+        armed_device.store(dev, std::memory_order_release);
+    }
+    const int row_tiles = M / kTileRows;
+    const int groups = (row_tiles + waves - 1) / waves;
+    hipLaunchKernelGGL(kernel, dim3(groups * split_k), dim3(waves * kWave), lds_bytes, stream,
                        static_cast<const u32x4*>(items), offsets, static_cast<const _Float16*>(B),
                        static_cast<_Float16*>(out), M, N, K, split_k);
     return static_cast<int>(hipGetLastError());
@@ -417,19 +500,23 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
 // Launchers called by the host logic.  Shapes are validated by the caller; all
 // pointers are device memory; everything is asynchronous on `stream`.
 
+// waves = waves per workgroup (1..8 for N <= 16, 1..4 above); stage_b != 0 stages the
+// activation slice in LDS (N <= 16 only); lds_bytes = waves * 16384 (+ slice bytes).
 extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offsets, const void* B, void* out, int M,
-                                int N, int K, int split_k)
+                                int N, int K, int split_k, int waves, int stage_b, unsigned lds_bytes)
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (N) {
         case 8:
-            return launch_spmm<1, true>(s, items, offsets, B, out, M, N, K, split_k);
+            return stage_b ? launch_spmm<1, true, true, 8>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes)
+                           : launch_spmm<1, true, false, 8>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes);
         case 16:
-            return launch_spmm<1, false>(s, items, offsets, B, out, M, N, K, split_k);
+            return stage_b ? launch_spmm<1, false, true, 8>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes)
+                           : launch_spmm<1, false, false, 8>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes);
         case 32:
-            return launch_spmm<2, false>(s, items, offsets, B, out, M, N, K, split_k);
+            return launch_spmm<2, false, false, 4>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes);
         case 64:
-            return launch_spmm<4, false>(s, items, offsets, B, out, M, N, K, split_k);
+            return launch_spmm<4, false, false, 4>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes);
         default:
             return static_cast<int>(hipErrorInvalidValue);
     }
