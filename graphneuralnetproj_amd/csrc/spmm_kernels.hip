@@ -40,10 +40,12 @@
 //     itself when Split_K == 1).
 //
 // Rule for the asynchronous loads: the compiler does not know that the outputs of
-// the load asm statements arrive later.  A slot's registers may therefore only
-// become dead after a wait that covers the slot's loads -- consume() performs such
-// a wait on every path -- otherwise the register allocator could hand a register
-// with a load still in flight to an address computation.
+// the load asm statements arrive later.  On every path, each destination register
+// of a load must therefore stay live until after a wait that covers the load:
+// land() waits and then names all registers of the slot as inputs of an (empty)
+// asm statement.  Without that, the register allocator could hand a register with
+// a load still in flight to some other value, which the landing load would then
+// overwrite.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -107,6 +109,14 @@ template<typename T>
 __device__ __forceinline__ void settle(T& x)
 {
     asm volatile("" : "+v"(x));
+}
+
+// A use of the register at this point and nothing else: keeps it reserved up to here
+// without creating a new value (which could make the compiler copy it elsewhere).
+template<typename T>
+__device__ __forceinline__ void pin(const T& x)
+{
+    asm volatile("" ::"v"(x));
 }
 
 // Four packed words -> four 16-bit LDS writes of the value (or of zero) at byte
@@ -205,6 +215,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
             wbase = i;
             const int idx = i + lane;
             wreg = toff[idx <= ntile ? idx : ntile];
+            settle(wreg);  // makes the compiler wait for this load here, on the rare path, not at the join below
         }
         begin = __builtin_amdgcn_readlane(wreg, i - wbase);
         end = __builtin_amdgcn_readlane(wreg, i + 1 - wbase);
@@ -306,25 +317,38 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
         }
     };
 
-    // Y = loads issued after this slot's that may stay in flight.
-    auto consume = [&](int slot, const Seg& s, auto younger) {
+    // Waits for every load of `slot` (at most Y younger ones may stay in flight) and keeps the
+    // slot's registers live up to that point, so none of them can be reused while a load into
+    // it is still on its way.
+    auto land = [&](int slot, auto younger) {
         constexpr int Y = decltype(younger)::value;
-        if (s.n == 0) {  // empty tile or past the end: only let the slot's loads land
-            wait_loads<Y>();
-            return;
+        wait_loads<Y>();
+        static_for<VPL>([&](auto uc) { pin(regs[slot][decltype(uc)::value]); });
+        if (!BLDS) {
+#pragma unroll
+            for (int cb = 0; cb < NB; cb++)
+#pragma unroll
+                for (int k = 0; k < 2; k++)
+                    settle(bfrag[slot][cb][k]);
         }
+    };
+
+    // Y = loads issued after this slot's that may stay in flight.  The slot's loads were issued
+    // a whole tile ago, so waiting for all of them up front costs nothing in steady state and
+    // keeps one unconditional wait on every path through the loop.
+    auto consume = [&](int slot, const Seg& s, auto younger) {
+        land(slot, younger);
+        if (s.n == 0)
+            return;  // empty tile or past the end
         static_for<VPL>([&](auto uc) {
             constexpr int u = decltype(uc)::value;
             if (u * kWave < s.n) {
-                wait_loads<Y + (L - 1 - u)>();
-                settle(regs[slot][u]);
                 if ((u + 1) * kWave <= s.n)
                     scatter_words<false>(regs[slot][u], vbase, vtwo, vzero);
                 else if (u * kWave + lane < s.n)  // the segment's last, partial chunk
                     scatter_words<false>(regs[slot][u], vbase, vtwo, vzero);
             }
         });
-        wait_loads<Y>();
         if (!s.last)
             return;  // more segments of this tile follow
         half8 bf[NB][2];
@@ -339,10 +363,8 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
 #pragma unroll
             for (int cb = 0; cb < NB; cb++)
 #pragma unroll
-                for (int k = 0; k < 2; k++) {
-                    settle(bfrag[slot][cb][k]);
+                for (int k = 0; k < 2; k++)
                     bf[cb][k] = bfrag[slot][cb][k];
-                }
         }
         // read the dense tile back and multiply; all reads of a pass are issued before its MFMAs
         constexpr int kPasses = NB == 1 ? 1 : 2;
@@ -403,7 +425,11 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
             if (held[0].tile >= ntile)
                 break;  // every later slot is past the end as well
         }
-        wait_loads<0>();
+        // the loads of the last (empty) issues are still in flight: let them land while their
+        // destination registers are still reserved
+#pragma unroll
+        for (int s = 0; s < D; s++)
+            land(s, std::integral_constant<int, 0>{});
     }
 
     // Epilogue.  acc[c][r][i] is output row r*16 + 4*q + i of this tile row for token
@@ -428,6 +454,9 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
                 *reinterpret_cast<half4*>(tile + l15 * kTokStride + (r * 16 + q * 4) * 2) = h;
             }
         }
+        // other lanes read what this lane wrote: the compiler must not move the reads above
+        // the writes (it reasons per lane), and the writes must have landed
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
         for (int i = 0; i < kTok / 4; i++) {
             const int e = i * kWave + lane;
@@ -438,24 +467,40 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
     }
 }
 
-// C[e] = fp16(sum over slabs of float(W[s][e])), 8 elements per thread.
-__global__ __launch_bounds__(256) void tcsl_reduce_kernel(_Float16* __restrict__ C, const _Float16* __restrict__ W,
-                                                         long mn8, long mn, int split_k)
+// C[e] = fp16(sum over slabs of float(W[s][e])) (csrc/Reduction_Kernel.cuh:36-46), 8 elements
+// per thread.  The slab loads of a thread are independent; they are issued eight at a time
+// so their latencies overlap (the reduction is latency bound: a few MB in all).
+__global__ __launch_bounds__(64) void tcsl_reduce_kernel(_Float16* __restrict__ C, const _Float16* __restrict__ W,
+                                                        long mn8, long mn, int split_k)
 {
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < mn8; i += (long)gridDim.x * blockDim.x) {
-        float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (int s = 0; s < split_k; s++) {
-            half8 w = *reinterpret_cast<const half8*>(W + (size_t)s * mn + i * 8);
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= mn8)
+        return;
+    const _Float16* w0 = W + i * 8;
+    float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    int s = 0;
+    for (; s + 8 <= split_k; s += 8) {
+        half8 w[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            w[u] = __builtin_nontemporal_load(reinterpret_cast<const half8*>(w0 + (size_t)(s + u) * mn));
+#pragma unroll
+        for (int u = 0; u < 8; u++)  // summed in slab order, as the reference does
 #pragma unroll
             for (int j = 0; j < 8; j++)
-                sum[j] += static_cast<float>(w[j]);
-        }
-        half8 o;
+                sum[j] += static_cast<float>(w[u][j]);
+    }
+    for (; s < split_k; s++) {
+        const half8 w = __builtin_nontemporal_load(reinterpret_cast<const half8*>(w0 + (size_t)s * mn));
 #pragma unroll
         for (int j = 0; j < 8; j++)
-            o[j] = static_cast<_Float16>(sum[j]);
-        *reinterpret_cast<half8*>(C + i * 8) = o;
+            sum[j] += static_cast<float>(w[j]);
     }
+    half8 o;
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+        o[j] = static_cast<_Float16>(sum[j]);
+    *reinterpret_cast<half8*>(C + i * 8) = o;
 }
 
 // Plain streaming copy, used only to calibrate hardware counters against a
@@ -525,12 +570,10 @@ extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offs
 extern "C" int tcsl_launch_reduce(void* stream, void* C, const void* W, long mn, int split_k)
 {
     const long mn8 = mn / 8;
-    long blocks = (mn8 + 255) / 256;
-    if (blocks > 4096)
-        blocks = 4096;
-    if (blocks < 1)
-        blocks = 1;
-    hipLaunchKernelGGL(tcsl_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+    const long blocks = (mn8 + 63) / 64;
+    if (blocks < 1 || blocks > 0x7fffffffL)
+        return static_cast<int>(hipErrorInvalidValue);
+    hipLaunchKernelGGL(tcsl_reduce_kernel, dim3((unsigned)blocks), dim3(64), 0, static_cast<hipStream_t>(stream),
                        static_cast<_Float16*>(C), static_cast<const _Float16*>(W), mn8, mn, split_k);
     return static_cast<int>(hipGetLastError());
 }

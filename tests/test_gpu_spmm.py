@@ -114,6 +114,117 @@ def test_uneven_and_oversized_split(spmm, oracle):
         assert_close(W, W_or)
 
 
+@pytest.mark.parametrize("M,K,N,split_k,sparsity", [
+    (640, 1024, 16, 2, 0.8),     # 5 tile rows: workgroups of several waves, the last one with idle waves
+    (896, 1792, 8, 4, 0.8),      # N = 8 with the activation slice staged in LDS
+    (128, 8192, 16, 1, 0.8),     # one unit of 128 tiles: the offsets window slides; slice too large to stage
+    (128, 12288, 8, 2, 0.9),     # 96-tile units with N = 8
+    (1152, 512, 16, 8, 0.75),    # one tile per unit
+    (384, 2048, 32, 3, 0.8),     # two column blocks, uneven batches (32 tiles over 3)
+    (256, 2048, 64, 2, 0.6),     # four column blocks, tiles longer than one register window
+    (2048, 256, 16, 2, 0.95),    # many tile rows, short K
+])
+def test_launch_shapes(spmm, oracle, M, K, N, split_k, sparsity):
+    """Shapes chosen to reach every launch plan of the main kernel: several waves per
+    workgroup with and without idle waves, staged and unstaged activations, long units."""
+    A, B, items, offsets = make_case(spmm, M, K, N, sparsity, seed=M + K + N)
+    C, W = run_gpu(spmm, items, offsets, B, M, N, K, split_k)
+    assert_close(C, oracle.gemm_f32(A, B))
+    C_or, W_or = oracle.spmm_splitk(items, offsets, B, M, N, K, split_k)
+    assert_close(C, C_or)
+    if split_k > 1:
+        assert_close(W, W_or)
+
+
+def test_partials_entry_point(spmm, oracle):
+    """SpMM_SplitK_Partials writes the same slabs SpMM_SplitK_API leaves in the workspace."""
+    import ctypes
+
+    torch = _torch()
+    M, K, N, split_k = 512, 1024, 16, 4
+    A, B, items, offsets = make_case(spmm, M, K, N, 0.8, seed=99)
+    dev = torch.device("cuda:0")
+    d_items = torch.from_numpy(items.view(np.int32).copy()).to(dev)
+    d_offs = torch.from_numpy(offsets.copy()).to(dev)
+    d_B = torch.from_numpy(B.view(np.int16).copy()).to(dev)
+    d_P = torch.full((split_k, N, M), float("nan"), dtype=torch.float16, device=dev)
+    lib = spmm.load_library()
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    rc = lib.SpMM_SplitK_Partials(None, p(d_items), p(d_offs), p(d_B), p(d_P), M, N, K, split_k)
+    assert rc == 0
+    torch.cuda.synchronize()
+    _, W_or = oracle.spmm_splitk(items, offsets, B, M, N, K, split_k)
+    assert_close(d_P.cpu().numpy(), W_or)
+    assert lib.SpMM_SplitK_Partials(None, p(d_items), p(d_offs), p(d_B), p(d_P), M, 24, K, split_k) != 0
+    assert lib.SpMM_SplitK_Partials(None, p(d_items), p(d_offs), p(d_B), None, M, N, K, split_k) != 0
+
+
+def test_repeated_calls_share_workspace(spmm, oracle):
+    """Back-to-back calls on one stream with one workspace (the caller contract) and different weights."""
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    M, K, N, split_k = 384, 768, 16, 3
+    cases = [make_case(spmm, M, K, N, 0.8, seed=500 + i) for i in range(3)]
+    d_W = torch.empty((split_k, N, M), dtype=torch.float16, device=dev)
+    outs = []
+    keep = []
+    for A, B, items, offsets in cases:
+        d_items = torch.from_numpy(items.view(np.int32).copy()).to(dev)
+        d_offs = torch.from_numpy(offsets.copy()).to(dev)
+        d_B = torch.from_numpy(B.view(np.int16).copy()).to(dev)
+        d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device=dev)
+        keep.append((d_items, d_offs, d_B))
+        spmm.SpMM_SplitK_API(torch.cuda.current_stream(), None, d_items, d_offs, d_B, d_C, M, N, K, d_W, split_k)
+        outs.append(d_C)
+    torch.cuda.synchronize()
+    for (A, B, items, offsets), d_C in zip(cases, outs):
+        assert_close(d_C.cpu().numpy(), oracle.gemm_f32(A, B))
+
+
+def test_full_size_properties(spmm, oracle):
+    """Headline shape (OPT-30B FFN1, 28672 x 7168, N=16, 80 %): checks that do not need the
+    full CPU product: linearity in the activations, a one-hot activation reproducing a
+    column of A exactly, and a row sample against the oracle."""
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    M, K, N = 28672, 7168, 16
+    split_k = spmm.SpMM_SuggestSplitK(M, N, K)
+    A = spmm.synth_weights(M, K, 0.8, False, seed=1234)
+    items, offsets = spmm.InitSparseMatrixA_API(A)
+    B1 = spmm.synth_activations(N, K, seed=1)
+    B2 = spmm.synth_activations(N, K, seed=2)
+    E = np.zeros((N, K), dtype=np.float16)
+    ks = np.random.default_rng(3).integers(0, K, N)
+    E[np.arange(N), ks] = 1.0
+    d_items = torch.from_numpy(items.view(np.int32)).to(dev)
+    d_offs = torch.from_numpy(offsets).to(dev)
+    d_W = torch.empty((split_k, N, M), dtype=torch.float16, device=dev)
+
+    def run(Bh):
+        d_B = torch.from_numpy(np.ascontiguousarray(Bh).view(np.int16)).to(dev)
+        d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device=dev)
+        spmm.SpMM_SplitK_API(None, None, d_items, d_offs, d_B, d_C, M, N, K, d_W, split_k)
+        torch.cuda.synchronize()
+        return d_C.cpu().numpy()
+
+    print(f"[gpu case] full size M={M} K={K} N={N} split_k={split_k}", flush=True)
+    C1, C2 = run(B1), run(B2)
+    # exact: one-hot activations pick columns of A (a single non-zero product per output)
+    CE = run(E)
+    assert np.array_equal(CE.view(np.uint16), (A[:, ks].T + np.float16(0)).view(np.uint16))
+    # linearity within rounding: A*(B1 + B2) = A*B1 + A*B2
+    Bs = (B1.astype(np.float32) + B2.astype(np.float32)).astype(np.float16)
+    Cs = run(Bs)
+    exact_sum = (Bs.astype(np.float32) == B1.astype(np.float32) + B2.astype(np.float32))
+    cols = np.flatnonzero(exact_sum.all(axis=1))  # tokens whose fp16 sum is exact
+    lin = C1.astype(np.float32) + C2.astype(np.float32)
+    if len(cols):
+        assert_close(Cs[cols], lin[cols])
+    # row sample against the oracle
+    rows = np.unique(np.concatenate([np.arange(128), np.arange(M - 128, M), np.random.default_rng(4).integers(0, M, 512)]))
+    assert_close(C1[:, rows], oracle.gemm_f32(np.ascontiguousarray(A[rows]), B1))
+
+
 def test_split1_leaves_workspace_alone(spmm):
     torch = _torch()
     M, K, N = 128, 128, 16
