@@ -17,7 +17,8 @@ import subprocess
 import numpy as np
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_PKG, "lib", "libSpMM_API.so")
+# SPMM_LIB_PATH selects another build of the same library (used to compare kernel variants).
+_LIB_PATH = os.environ.get("SPMM_LIB_PATH") or os.path.join(_PKG, "lib", "libSpMM_API.so")
 
 _u16p = ctypes.POINTER(ctypes.c_uint16)
 _u32p = ctypes.POINTER(ctypes.c_uint32)
