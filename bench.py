@@ -30,6 +30,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch of the main kernel from rocprofv3 counter runs (FETCH_SIZE and WRITE_SIZE,
+# each scaled by what the same counter reads for a copy kernel of known size); summaries of
+# those runs are kept under profiles/.  Keyed by (workload, N, split_k); None where not measured.
+MEASURED_TRAFFIC_BYTES = {
+    ("opt30b_ffn1", 16, 8): 175.50e6,
+}
 FP16_MFMA_PEAK_TFLOPS = 2500.0
 
 WORKLOADS = {
@@ -38,7 +44,10 @@ WORKLOADS = {
     "opt30b_ffn2": (7168, 28672, 16, 0.8, False),
     "opt30b_qkv": (21504, 7168, 16, 0.8, False),
     "opt30b_outproj": (7168, 7168, 16, 0.8, False),
+    "opt66b_qkv": (27648, 9216, 16, 0.8, False),
+    "opt66b_outproj": (9216, 9216, 16, 0.8, False),
     "opt66b_ffn1": (36864, 9216, 16, 0.8, False),
+    "opt66b_ffn2": (9216, 36864, 16, 0.8, False),
     "config1": (1024, 1024, 8, 0.8, False),
 }
 
@@ -72,6 +81,16 @@ def cpu_baseline(A, B, M, N, K, max_seconds=30.0):
     O.gemm_f32(A[:rows], B)
     t_gemm = (time.perf_counter() - t0) * (M / rows)
     flops = 2.0 * M * N * K
+
+    # the same GEMM spread over the host's cores by 128-row blocks (ctypes releases the GIL)
+    from concurrent.futures import ThreadPoolExecutor
+
+    threads = max(1, min(16, os.cpu_count() or 1))
+    blocks = [(r, min(r + 128, rows)) for r in range(0, rows, 128)]
+    t0 = time.perf_counter()
+    with ThreadPoolExecutor(threads) as pool:
+        list(pool.map(lambda rb: O.gemm_f32(A[rb[0]:rb[1]], B), blocks))
+    t_gemm_mt = (time.perf_counter() - t0) * (M / rows)
     return {
         "value": flops / t_gemm / 1e12,
         "unit": "TFLOPS",
@@ -83,6 +102,7 @@ def cpu_baseline(A, B, M, N, K, max_seconds=30.0):
         "encode_s": t_enc,
         "encode_kind": enc_kind,
         "value_with_encode": flops / (t_gemm + t_enc) / 1e12,
+        "all_cores": {"value": flops / t_gemm_mt / 1e12, "unit": "TFLOPS", "cores": threads, "gemm_s": t_gemm_mt},
     }
 
 
@@ -100,6 +120,9 @@ def main():
     ap.add_argument("--copies", type=int, default=0, help="distinct HBM copies of the weight (0 = enough for > 640 MB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--calibration-copies", type=int, default=0,
+                    help="after the timed regions, run this many device-to-device copies of the compressed "
+                         "weight (SpMM_CalibrationCopy): a kernel of known traffic for scaling byte counters")
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -204,6 +227,13 @@ def main():
     lib.SpMM_EventDestroy(ev1)
     torch.cuda.synchronize()
 
+    for i in range(args.calibration_copies):
+        src, dst = d_items[i % copies], d_items[(i + 1) % copies]  # all copies hold the same bytes
+        rc = lib.SpMM_CalibrationCopy(sptr, ctypes.c_void_p(dst.data_ptr()), ctypes.c_void_p(src.data_ptr()), a_bytes)
+        if rc:
+            raise RuntimeError(f"SpMM_CalibrationCopy -> {rc}")
+    torch.cuda.synchronize()
+
     flops = 2.0 * M * N * K
     tflops = flops / (ms_per_step * 1e-3) / 1e12
     kernel_gbps = a_bytes / (kernel_ms_avg * 1e-3) / 1e9
@@ -225,6 +255,8 @@ def main():
                          f"{'Beta(2,8) row-skewed' if skew else 'Bernoulli'} sparsity, fp16, fp32 accumulate"),
             "split_k": split_k,
             "compressed_bytes": a_bytes,
+            "total_algorithmic_bytes": (a_bytes + 4 * len(offsets) + 2 * K * N + 2 * M * N
+                                        + (4 * split_k * M * N if split_k > 1 else 0)),
             "weight_copies_rotated": copies,
             "layout": "B[N][K], C[N][M]",
         },
@@ -237,7 +269,8 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": kernel_gbps / HBM_PEAK_GBPS,
-            "traffic": None,
+            "traffic": (MEASURED_TRAFFIC_BYTES.get((args.workload, N, split_k))
+                        if sparsity == 0.8 and not skew else None),
             "kernel": "tcsl_spmm_kernel",
             "kernel_ms_avg": kernel_ms_avg,
             "algorithmic_bytes_per_launch": a_bytes,
