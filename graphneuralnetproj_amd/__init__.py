@@ -2,7 +2,9 @@
 from .spmm_api import (  # noqa: F401
     GenSparseMatrixBinFile,
     InitSparseMatrixA_API,
+    SpMM_PlanLaunch,
     SpMM_SplitK_API,
+    SpMM_SplitK_API_Planned,
     SpMM_SuggestSplitK,
     SpMMError,
     build_library,

@@ -1,0 +1,204 @@
+// Picks the launch shape of the main kernel: which of its two workgroup layouts, how many
+// waves per workgroup, and (for SpMM_SuggestSplitK) how many split-K batches.
+//
+// The reference fixes one block shape and tunes Split_K per matrix by hand
+// (kernel_benchmark/benchmark.sh:15, end2end_inference/ft_tools/huggingface_opt_convert_Phase2.py:20).
+// Here the choice is made by a small analytic model of an MI355X (256 compute units, one
+// workgroup slot set per unit limited by LDS and registers), fitted to a sweep of about 2500
+// measured (shape, N, plan) points on OPT-30B/66B layer shapes at 80 % sparsity, backed by a
+// table of the measured optimum for those shapes themselves.
+#include "launch_plan.h"
+
+#include <cmath>
+
+#include "tiled_csl_format.h"
+
+namespace tcsl {
+
+namespace {
+
+constexpr long kLdsPerCu = 160 * 1024;
+constexpr long kTileLds = 16384;   // dense fp16 image of one 128x64 tile
+constexpr int kCUs = 256;
+
+// Fitted constants (microseconds, bytes per microsecond).
+constexpr double kLaunchUs = 2.87;          // fixed cost of the main kernel
+constexpr double kTileBytes = 6558.0;       // one tile at 80 % sparsity
+constexpr double kChipBytesPerUs = 7.0e6;   // whole-chip stream rate
+constexpr double kCuBytesPerUs = 38.3e3;    // what one compute unit can pull on its own
+constexpr double kWaveTileUs = 0.712;       // a lone wave's turnaround per tile (latency bound)
+constexpr double kMfmaTileUs = 0.174;       // serial MFMA + LDS time per tile and 16-token block
+constexpr double kRoundUs = 3.61;           // start-up and drain of one round of workgroups
+constexpr double kNorm = 3.65;              // exponent that blends the three bounds
+constexpr double kCrowdPenalty = 0.072;     // per resident wave above kCrowdWaves on a unit
+constexpr double kCrowdWaves = 7.0;
+constexpr double kGlobalBPenalty = 0.154;   // mode 0, N <= 16, slice not staged
+constexpr double kModeKPenalty = 0.051;     // mode 1: activations from L2, reduction in LDS
+constexpr double kReduceUs = 3.14;          // fixed cost of the reduction kernel
+constexpr double kReduceBytesPerUs = 4.75e6;
+
+int column_blocks(int N)
+{
+    return N <= 16 ? 1 : N / 16;
+}
+
+int max_waves(int N)
+{
+    return N <= 32 ? 8 : 4;  // registers: two waves per SIMD up to N = 32, one at N = 64
+}
+
+// Measured optimum for the layer shapes of OPT-30B and OPT-66B (80 % sparsity):
+// {M, K, N, Split_K, mode, waves, stage_b}.
+struct Tuned {
+    int M, K, N, split_k, mode, waves, stage_b;
+};
+constexpr Tuned kTuned[] = {
+#include "tuned_plans.inc"
+};
+
+const Tuned* find_tuned(int M, int N, int K)
+{
+    for (const Tuned& t : kTuned)
+        if (t.M == M && t.K == K && t.N == N)
+            return &t;
+    return nullptr;
+}
+
+}  // namespace
+
+bool complete_plan(int N, int K, int split_k, LaunchPlan& p)
+{
+    if (N != 8 && N != 16 && N != 32 && N != 64)
+        return false;
+    if (split_k < 1 || p.waves < 1 || p.waves > max_waves(N))
+        return false;
+    const int nb = column_blocks(N);
+    const long nkb = K / kTileCols;
+    const long tiles = (nkb - 1) / split_k + 1;  // tiles of the longest batch
+    long lds = p.waves * kTileLds;
+    if (p.mode == 0) {
+        if (p.stage_b) {
+            if (nb != 1)
+                return false;
+            lds += tiles * (N == 8 ? 8 : 16) * 128;
+        }
+    } else if (p.mode == 1) {
+        if (p.stage_b)
+            return false;
+        const long red = 8L * p.waves * nb * 1024;  // fp32 accumulators of all waves
+        if (red > lds)
+            lds = red;
+    } else {
+        return false;
+    }
+    if (lds > kLdsPerCu)
+        return false;
+    p.lds_bytes = static_cast<unsigned>(lds);
+    return true;
+}
+
+double plan_cost_us(int M, int N, int K, int split_k, const LaunchPlan& p)
+{
+    const long row_tiles = M / kTileRows;
+    const long nkb = K / kTileCols;
+    const int nb = column_blocks(N);
+    const int W = p.waves;
+    const long batch_tiles = (nkb - 1) / split_k + 1;
+    long wgs, t;  // workgroups; tiles per wave
+    if (p.mode == 0) {
+        wgs = (row_tiles + W - 1) / W * split_k;
+        t = batch_tiles;
+    } else {
+        wgs = row_tiles * split_k;
+        t = (batch_tiles + W - 1) / W;
+    }
+    long fit = kLdsPerCu / (p.lds_bytes ? p.lds_bytes : 1);
+    if (fit > max_waves(N) / W)
+        fit = max_waves(N) / W;
+    if (fit < 1)
+        fit = 1;
+    const long slots = kCUs * fit;
+    const double tau_chip = kTileBytes / kChipBytesPerUs;
+    const double tau_cu = kTileBytes / kCuBytesPerUs;
+    const double tau_wave = kWaveTileUs + kMfmaTileUs * nb;
+    double total = kLaunchUs;
+    for (long left = wgs; left > 0;) {
+        const long n = left < slots ? left : slots;
+        left -= n;
+        const long per_cu = (n + kCUs - 1) / kCUs;
+        const double crowd = static_cast<double>(per_cu * W) - kCrowdWaves;
+        const double chip = static_cast<double>(n) * W * t * tau_chip * (1.0 + (crowd > 0 ? kCrowdPenalty * crowd : 0.0));
+        const double lat = kRoundUs + t * tau_wave;
+        const double cu = static_cast<double>(per_cu) * W * t * tau_cu;
+        total += std::pow(std::pow(chip, kNorm) + std::pow(lat, kNorm) + std::pow(cu, kNorm), 1.0 / kNorm);
+    }
+    if (p.mode == 0 && nb == 1 && !p.stage_b)
+        total *= 1.0 + kGlobalBPenalty;
+    if (p.mode == 1)
+        total *= 1.0 + kModeKPenalty;
+    if (split_k > 1)
+        total += kReduceUs + (2.0 * split_k + 1.0) * M * N * 2.0 / kReduceBytesPerUs;
+    return total;
+}
+
+LaunchPlan plan_launch(int M, int N, int K, int split_k, double* cost_us)
+{
+    if (const Tuned* t = find_tuned(M, N, K)) {
+        LaunchPlan p{t->mode, t->waves, t->stage_b, 0};
+        if (t->split_k == split_k && complete_plan(N, K, split_k, p)) {
+            if (cost_us)
+                *cost_us = plan_cost_us(M, N, K, split_k, p);
+            return p;
+        }
+    }
+    LaunchPlan best{0, 1, 0, static_cast<unsigned>(kTileLds)};
+    double best_cost = -1.0;
+    for (int mode = 0; mode <= 1; mode++)
+        for (int w = 1; w <= max_waves(N); w++)
+            for (int stage = 0; stage <= (mode == 0 ? 1 : 0); stage++) {
+                LaunchPlan p{mode, w, stage, 0};
+                if (!complete_plan(N, K, split_k, p))
+                    continue;
+                const double c = plan_cost_us(M, N, K, split_k, p);
+                if (best_cost < 0 || c < best_cost) {
+                    best = p;
+                    best_cost = c;
+                }
+            }
+    if (cost_us)
+        *cost_us = best_cost;
+    return best;
+}
+
+int suggest_split_k(int M, int N, int K, LaunchPlan* plan)
+{
+    if (const Tuned* t = find_tuned(M, N, K)) {
+        LaunchPlan p{t->mode, t->waves, t->stage_b, 0};
+        if (complete_plan(N, K, t->split_k, p)) {
+            if (plan)
+                *plan = p;
+            return t->split_k;
+        }
+    }
+    const long nkb = K / kTileCols > 0 ? K / kTileCols : 1;
+    int best = 1;
+    double best_cost = -1.0;
+    LaunchPlan best_plan{0, 1, 0, static_cast<unsigned>(kTileLds)};
+    for (long s = 1; s <= 32 && s <= nkb; s++) {
+        const long tiles = (nkb + s - 1) / s;
+        if (s > 1 && tiles * (s - 1) >= nkb)
+            continue;  // a split that leaves the last batch empty
+        double c = 0.0;
+        const LaunchPlan p = plan_launch(M, N, K, static_cast<int>(s), &c);
+        if (best_cost < 0 || c < best_cost - 1e-9) {
+            best = static_cast<int>(s);
+            best_cost = c;
+            best_plan = p;
+        }
+    }
+    if (plan)
+        *plan = best_plan;
+    return best;
+}
+
+}  // namespace tcsl

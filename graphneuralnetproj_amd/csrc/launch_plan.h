@@ -1,0 +1,29 @@
+// Launch shape of the main kernel and the cost model that picks it.  Host only.
+#pragma once
+
+namespace tcsl {
+
+// mode 0: the W waves of a workgroup take W consecutive 128-row tile rows of one split-K
+//         batch (stage_b: the batch's activation slice is staged in LDS and shared);
+// mode 1: the W waves of a workgroup split the batch of one tile row among themselves and
+//         add their accumulators up in LDS.
+struct LaunchPlan {
+    int mode;
+    int waves;
+    int stage_b;
+    unsigned lds_bytes;
+};
+
+// True (and lds_bytes filled in) when the kernels can run this shape.
+bool complete_plan(int N, int K, int split_k, LaunchPlan& p);
+
+// Estimated time in microseconds of SpMM_SplitK_API (main kernel + reduction) with this plan.
+double plan_cost_us(int M, int N, int K, int split_k, const LaunchPlan& p);
+
+// Best plan for a given Split_K; *cost_us (optional) receives its estimate.
+LaunchPlan plan_launch(int M, int N, int K, int split_k, double* cost_us);
+
+// Best Split_K in 1..32 (with its plan) for the shape.
+int suggest_split_k(int M, int N, int K, LaunchPlan* plan);
+
+}  // namespace tcsl

@@ -6,11 +6,12 @@
 #include <cstdlib>
 
 #include "../../include/SpMM_API.h"
+#include "launch_plan.h"
 #include "tiled_csl_format.h"
 
 extern "C" {
 int tcsl_launch_spmm(void* stream, const void* items, const int* offsets, const void* B, void* out, int M, int N,
-                     int K, int split_k, int waves, int stage_b, unsigned lds_bytes);
+                     int K, int split_k, int mode, int waves, int stage_b, unsigned lds_bytes);
 int tcsl_launch_reduce(void* stream, void* C, const void* W, long mn, int split_k);
 int tcsl_launch_copy(void* stream, void* dst, const void* src, long bytes);
 void* tcsl_event_create(void);
@@ -47,61 +48,36 @@ extern "C" const char* SpMM_GetErrorString(int code)
 
 namespace {
 
-// Launch shape of the main kernel: W waves per workgroup (each wave owns one 128-row tile
-// row of one batch), and whether the batch's activation slice is staged in LDS.
-struct LaunchPlan {
-    int waves;
-    int stage_b;
-    unsigned lds_bytes;
-};
-
-LaunchPlan plan_launch(int M, int N, int K, int Split_K)
+// Plans are a pure function of the shape; the last few are remembered per thread so that a
+// decode loop cycling over a handful of layer shapes never re-runs the model.
+tcsl::LaunchPlan cached_plan(int M, int N, int K, int Split_K)
 {
-    constexpr long kLds = 160 * 1024, kTile = 16384, kCUs = 256;
-    const long row_tiles = M / tcsl::kTileRows;
-    const long nkb = K / tcsl::kTileCols;
-    const long tiles = (nkb - 1) / Split_K + 1;  // tiles of the longest batch
-    if (N > 16)  // wide accumulators: one wave per workgroup, activations from global memory
-        return LaunchPlan{1, 0, static_cast<unsigned>(kTile)};
-    const long slice = tiles * (N == 8 ? 8 : 16) * 128;  // staged activation bytes
-    // Pick W: the busiest compute unit runs ceil(workgroups / 256) workgroups of W waves of
-    // `tiles` tiles each, and pulls its stream at full rate only with about seven waves
-    // resident.  Ties go to the larger W (more waves share one staged slice).
-    LaunchPlan best{1, 0, static_cast<unsigned>(kTile)};
-    double best_cost = 0.0;
-    for (int w = 1; w <= 8; w++) {
-        for (int stage = 0; stage <= 1; stage++) {
-            const long lds = w * kTile + (stage ? slice : 0);
-            if (lds > kLds)
-                continue;
-            const long wgs = (row_tiles + w - 1) / w * Split_K;
-            long fit = kLds / lds;  // workgroups resident per compute unit
-            if (fit > 8 / w)
-                fit = 8 / w;        // eight waves per compute unit at this kernel's register use
-            const long per_cu = (wgs + kCUs - 1) / kCUs;
-            const long resident = (per_cu < fit ? per_cu : fit) * w;
-            double cost = static_cast<double>(per_cu) * w * tiles * (resident < 7 ? 7.0 / resident : 1.0);
-            if (!stage)
-                cost *= 1.03;  // activations re-fetched through L2 for every tile
-            if (best_cost == 0.0 || cost <= best_cost * (1.0 + 1e-9)) {
-                best = LaunchPlan{w, stage, static_cast<unsigned>(lds)};
-                best_cost = cost;
-            }
-        }
-    }
-    return best;
+    struct Entry {
+        int M, N, K, S;
+        tcsl::LaunchPlan plan;
+    };
+    constexpr int kEntries = 16;
+    thread_local Entry cache[kEntries] = {};
+    thread_local int next = 0;
+    for (const Entry& e : cache)
+        if (e.M == M && e.N == N && e.K == K && e.S == Split_K)
+            return e.plan;
+    const tcsl::LaunchPlan p = tcsl::plan_launch(M, N, K, Split_K, nullptr);
+    cache[next] = Entry{M, N, K, Split_K, p};
+    next = (next + 1) % kEntries;
+    return p;
 }
 
 int launch_main(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* out, int M, int N,
-                int K, int Split_K)
+                int K, int Split_K, const tcsl::LaunchPlan* forced)
 {
-    const LaunchPlan p = plan_launch(M, N, K, Split_K);
-    return tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, out, M, N, K, Split_K, p.waves, p.stage_b,
+    const tcsl::LaunchPlan p = forced ? *forced : cached_plan(M, N, K, Split_K);
+    return tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, out, M, N, K, Split_K, p.mode, p.waves, p.stage_b,
                             p.lds_bytes);
 }
 
 int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* C, int M, int N,
-                int K, void* Reduction_Workspace, int Split_K, void* ev_begin, void* ev_end);
+                int K, void* Reduction_Workspace, int Split_K, void* ev_begin, void* ev_end, const tcsl::LaunchPlan* forced);
 }
 
 extern "C" int SpMM_SplitK_API(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets,
@@ -109,7 +85,39 @@ extern "C" int SpMM_SplitK_API(void* stream, const void* A, const void* Compress
 {
     (void)A;
     return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, nullptr,
-                       nullptr);
+                       nullptr, nullptr);
+}
+
+extern "C" int SpMM_SplitK_API_Planned(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
+                                       void* C, int M, int N, int K, void* Reduction_Workspace, int Split_K, int Mode,
+                                       int Waves, int StageB)
+{
+    tcsl::LaunchPlan p{Mode, Waves, StageB, 0};
+    if (!tcsl::complete_plan(N, K > 0 ? K : 64, Split_K, p))
+        return tcsl_error_invalid_value();
+    return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, nullptr,
+                       nullptr, &p);
+}
+
+extern "C" int SpMM_PlanLaunch(int M, int N, int K, int Split_K, int* Mode, int* Waves, int* StageB, int* LdsBytes,
+                               double* EstimatedUs)
+{
+    if ((N != 8 && N != 16 && N != 32 && N != 64) || M <= 0 || K <= 0 || M % tcsl::kTileRows != 0 ||
+        K % tcsl::kTileCols != 0 || Split_K < 1)
+        return -1;
+    double cost = 0.0;
+    const tcsl::LaunchPlan p = tcsl::plan_launch(M, N, K, Split_K, &cost);
+    if (Mode)
+        *Mode = p.mode;
+    if (Waves)
+        *Waves = p.waves;
+    if (StageB)
+        *StageB = p.stage_b;
+    if (LdsBytes)
+        *LdsBytes = static_cast<int>(p.lds_bytes);
+    if (EstimatedUs)
+        *EstimatedUs = cost;
+    return 0;
 }
 
 extern "C" int SpMM_SplitK_API_Events(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets,
@@ -118,7 +126,7 @@ extern "C" int SpMM_SplitK_API_Events(void* stream, const void* A, const void* C
 {
     (void)A;
     return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, KernelBegin,
-                       KernelEnd);
+                       KernelEnd, nullptr);
 }
 
 extern "C" int SpMM_SplitK_Partials(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
@@ -131,7 +139,7 @@ extern "C" int SpMM_SplitK_Partials(void* stream, const void* Compressed_A, cons
         return tcsl_error_invalid_value();
     if (!Compressed_A || !TileOffsets || !B || !Partials)
         return tcsl_error_invalid_value();
-    return launch_main(stream, Compressed_A, TileOffsets, B, Partials, M, N, K, Split_K);
+    return launch_main(stream, Compressed_A, TileOffsets, B, Partials, M, N, K, Split_K, nullptr);
 }
 
 extern "C" void* SpMM_EventCreate(void)
@@ -157,7 +165,8 @@ extern "C" float SpMM_EventElapsedMs(void* start, void* stop)
 namespace {
 
 int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* C, int M, int N,
-                int K, void* Reduction_Workspace, int Split_K, void* ev_begin, void* ev_end)
+                int K, void* Reduction_Workspace, int Split_K, void* ev_begin, void* ev_end,
+                const tcsl::LaunchPlan* forced)
 {
     if (N != 8 && N != 16 && N != 32 && N != 64) {
         std::printf("MM_Sparse_API Error: Unsupported N dimension %d!\n", N);
@@ -172,7 +181,7 @@ int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, 
         std::fprintf(stderr, "SpMM_SplitK_API: null device pointer\n");
         return tcsl_error_invalid_value();
     }
-    // the launch grid is (M/128) * Split_K single-wave workgroups
+    // the launch grid is at most (M/128) * Split_K workgroups
     if (static_cast<long>(M / tcsl::kTileRows) * Split_K > 0x7fffffffL) {
         std::fprintf(stderr, "SpMM_SplitK_API: Split_K=%d too large for M=%d\n", Split_K, M);
         return tcsl_error_invalid_value();
@@ -181,7 +190,8 @@ int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, 
     int rc = 0;
     if (ev_begin && (rc = tcsl_event_record(ev_begin, stream)) != 0)
         return rc;
-    rc = launch_main(stream, Compressed_A, TileOffsets, B, Split_K == 1 ? C : Reduction_Workspace, M, N, K, Split_K);
+    rc = launch_main(stream, Compressed_A, TileOffsets, B, Split_K == 1 ? C : Reduction_Workspace, M, N, K, Split_K,
+                     forced);
     if (rc != 0)
         return rc;
     if (ev_end && (rc = tcsl_event_record(ev_end, stream)) != 0)
@@ -194,33 +204,10 @@ int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, 
 
 extern "C" int SpMM_SuggestSplitK(int M, int N, int K)
 {
-    if (M <= 0 || K <= 0 || N <= 0)
+    if (M <= 0 || K <= 0 || (N != 8 && N != 16 && N != 32 && N != 64))
         return 1;
-    // One wave per (128-row tile row, batch), spread over 256 compute units.  The stream a
-    // compute unit has to pull is the sum of its waves' tiles, and it needs about seven
-    // resident waves to pull at full rate, so the estimate to minimise is
-    //   max(ceil(units / 256), 7) * tiles_per_unit    busiest unit's share of the weight stream
-    // + units / 256 * slab_cost                       partial sums written, then read by the reduction
-    // in units of one 80 %-sparse tile (about 6.5 KB); ties go to the smaller split.
-    const long row_tiles = (M + tcsl::kTileRows - 1) / tcsl::kTileRows;
-    const long nkb = K / tcsl::kTileCols > 0 ? K / tcsl::kTileCols : 1;
-    const double slab_cost = 2.0 * tcsl::kTileRows * N * 2.0 / 6554.0;
-    int best = 1;
-    double best_cost = 0.0;
-    for (long s = 1; s <= 32 && s <= nkb; s++) {
-        const long tiles = (nkb + s - 1) / s;
-        if (s > 1 && (tiles < 2 || tiles * (s - 1) >= nkb))
-            continue;  // batches of one tile, or a split that leaves the last batch empty
-        const long units = row_tiles * s;
-        const long waves_per_cu = (units + 255) / 256;
-        const double cost = static_cast<double>(waves_per_cu > 7 ? waves_per_cu : 7) * tiles +
-                            (s > 1 ? units / 256.0 * slab_cost : 0.0);
-        if (s == 1 || cost < best_cost - 1e-9) {
-            best = static_cast<int>(s);
-            best_cost = cost;
-        }
-    }
-    return best;
+    return tcsl::suggest_split_k(M - M % tcsl::kTileRows > 0 ? M - M % tcsl::kTileRows : tcsl::kTileRows, N,
+                                 K - K % tcsl::kTileCols > 0 ? K - K % tcsl::kTileCols : tcsl::kTileCols, nullptr);
 }
 
 extern "C" void SpMM_SynthWeights(uint16_t* A_h, int M, int K, double sparsity, int row_skewed, uint64_t seed)

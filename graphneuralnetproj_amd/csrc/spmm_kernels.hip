@@ -156,7 +156,7 @@ __device__ __forceinline__ void clear_tile(uint8_t* tile, int lane)
 // and dropped); BLDS = the batch's activation slice is staged in LDS; MAXW bounds W and
 // with it the registers a wave may use.
 // Dynamic LDS: W tiles of 16 KiB, then (BLDS) tiles_per_batch * tokens * 128 bytes.
-template<int NB, bool HALF, bool BLDS, int MAXW>
+template<int NB, bool HALF, bool BLDS, bool KSPLIT, int MAXW>
 __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __restrict__ items,
                                                                 const int* __restrict__ offsets,
                                                                 const _Float16* __restrict__ B,
@@ -170,13 +170,14 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
     constexpr int kSeg = VPL * kWave;             // vectors per segment
     constexpr int NTOK = HALF ? 8 : NB * 16;      // tokens in the staged slice
 
+    static_assert(!(KSPLIT && BLDS), "a workgroup that splits K shares no activation slice");
     const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // uniform, and known to be
     const int W = blockDim.x / kWave;
     const int row_tiles = M / kTileRows;
-    const int groups = (row_tiles + W - 1) / W;
+    const int groups = KSPLIT ? row_tiles : (row_tiles + W - 1) / W;
     const int batch = blockIdx.x / groups;
-    const int rt = (blockIdx.x % groups) * W + wave;
+    const int rt = KSPLIT ? blockIdx.x % groups : (blockIdx.x % groups) * W + wave;
     const bool active = rt < row_tiles;
     // split-K bookkeeping of the reference (csrc/SpMM_Kernel.cuh:312-320), clamped to the matrix
     const int nkb = K / kTileCols;
@@ -185,7 +186,15 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
     kb0 = kb0 < nkb ? kb0 : nkb;
     int kb1 = kb0 + avg;
     kb1 = kb1 < nkb ? kb1 : nkb;
-    const int ntile = kb1 - kb0;  // tiles of this unit
+    if (KSPLIT) {
+        // The batch's tiles are dealt to the W waves in contiguous runs.  (Dealing them round
+        // robin, so that the workgroup reads one contiguous stretch at a time, measured slower.)
+        const int run = (kb1 - kb0 + W - 1) / W;
+        kb0 += wave * run;
+        kb0 = kb0 < kb1 ? kb0 : kb1;
+        kb1 = kb0 + run < kb1 ? kb0 + run : kb1;
+    }
+    const int ntile = kb1 - kb0;  // tiles of this wave
     uint8_t* const tile = lds + wave * kTileBytes;
     uint8_t* const bslice = lds + W * kTileBytes;  // [tile][token][8 granules of 16 B at position g ^ (token & 7)]
 
@@ -207,11 +216,11 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
         clear_tile(tile, lane);
     if (BLDS)
         __syncthreads();  // the only barrier: every wave of the workgroup reaches it
-    if (!active)
+    if (!KSPLIT && !active)
         return;
 
     auto tile_range = [&](int i, int& begin, int& end) {  // 0 <= i < ntile
-        if (i + 1 - wbase >= kWave) {  // slide the window (units longer than 63 tiles only)
+        if (i + 1 - wbase >= kWave) {  // slide the window (more than 63 tiles per wave only)
             wbase = i;
             const int idx = i + lane;
             wreg = toff[idx <= ntile ? idx : ntile];
@@ -440,9 +449,42 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
     // c*16 + l15; the output keeps one contiguous M vector per token.  The block goes through
     // the wave's LDS tile as [token][128 rows] (token stride padded to 272 B) so that the
     // global stores are 16 bytes per lane with 16 lanes covering a token's 256 bytes.
+    _Float16* oslab = out + (size_t)batch * M * N + (size_t)rt * kTileRows;
+    if (KSPLIT) {
+        // Sum the W waves' accumulators through LDS, in wave order.  Layout: [row block r]
+        // [source wave][column block c][lane] x 16 bytes; wave w then owns row blocks w, w + W, ...
+        f32x4* const red = reinterpret_cast<f32x4*>(lds);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's last clearing writes
+        __syncthreads();                                      // every wave is done with its tile
+#pragma unroll
+        for (int r = 0; r < 8; r++)
+#pragma unroll
+            for (int c = 0; c < NB; c++)
+                red[((r * W + wave) * NB + c) * kWave + lane] = acc[c][r];
+        __syncthreads();
+        for (int r = wave; r < 8; r += W) {
+#pragma unroll
+            for (int c = 0; c < NB; c++) {
+                f32x4 sum = red[((r * W) * NB + c) * kWave + lane];
+                for (int w = 1; w < W; w++) {
+                    const f32x4 v = red[((r * W + w) * NB + c) * kWave + lane];
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        sum[i] += v[i];
+                }
+                half4 h;
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    h[i] = static_cast<_Float16>(sum[i]);
+                // rows r*16 + 4*q .. +3 of token c*16 + l15: the four q-lanes of a token cover 32 bytes
+                if (!(HALF && l15 >= 8))
+                    *reinterpret_cast<half4*>(oslab + (size_t)(c * 16 + l15) * M + r * 16 + q * 4) = h;
+            }
+        }
+        return;
+    }
     constexpr int kTokStride = 272;
     constexpr int kTok = HALF ? 8 : 16;
-    _Float16* oslab = out + (size_t)batch * M * N + (size_t)rt * kTileRows;
 #pragma unroll
     for (int c = 0; c < NB; c++) {
         // the clearing writes of the last tile (inline asm, unknown to the compiler's own
@@ -515,13 +557,13 @@ __global__ __launch_bounds__(256) void tcsl_copy_kernel(u32x4* __restrict__ dst,
         dst[i] = src[i];
 }
 
-template<int NB, bool HALF, bool BLDS, int MAXW>
+template<int NB, bool HALF, bool BLDS, bool KSPLIT, int MAXW>
 int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const void* B, void* out, int M, int N,
                 int K, int split_k, int waves, unsigned lds_bytes)
 {
     if (waves < 1 || waves > MAXW || lds_bytes > kMaxLdsBytes)
         return static_cast<int>(hipErrorInvalidValue);
-    auto kernel = tcsl_spmm_kernel<NB, HALF, BLDS, MAXW>;
+    auto kernel = tcsl_spmm_kernel<NB, HALF, BLDS, KSPLIT, MAXW>;
     // more than 64 KiB of dynamic LDS has to be allowed once per kernel (per device, re-armed lazily)
     static std::atomic<int> armed_device{-1};
     int dev = 0;
@@ -536,7 +578,7 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
         armed_device.store(dev, std::memory_order_release);
     }
     const int row_tiles = M / kTileRows;
-    const int groups = (row_tiles + waves - 1) / waves;
+    const int groups = KSPLIT ? row_tiles : (row_tiles + waves - 1) / waves;
     hipLaunchKernelGGL(kernel, dim3(groups * split_k), dim3(waves * kWave), lds_bytes, stream,
                        static_cast<const u32x4*>(items), offsets, static_cast<const _Float16*>(B),
                        static_cast<_Float16*>(out), M, N, K, split_k);
@@ -549,26 +591,36 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
 // Launchers called by the host logic.  Shapes are validated by the caller; all
 // pointers are device memory; everything is asynchronous on `stream`.
 
-// waves = waves per workgroup (1..8 for N <= 16, 1..4 above); stage_b != 0 stages the
-// activation slice in LDS (N <= 16 only); lds_bytes = waves * 16384 (+ slice bytes).
+// mode 0: the W waves of a workgroup take W consecutive tile rows of one batch (and, with
+//         stage_b != 0 and N <= 16, share the batch's activation slice in LDS);
+// mode 1: the W waves of a workgroup split the batch of one tile row among themselves and
+//         add their results up in LDS (stage_b must be 0).
+// waves = 1..8 for N <= 16, 1..4 above; lds_bytes = what the mode needs (the host plans it).
 extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offsets, const void* B, void* out, int M,
-                                int N, int K, int split_k, int waves, int stage_b, unsigned lds_bytes)
+                                int N, int K, int split_k, int mode, int waves, int stage_b, unsigned lds_bytes)
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (mode != 0 && mode != 1)
+        return static_cast<int>(hipErrorInvalidValue);
+    if (mode == 1 && stage_b)
+        return static_cast<int>(hipErrorInvalidValue);
+#define TCSL_GO(NB, HALF, BLDS, KS, MAXW) \
+    launch_spmm<NB, HALF, BLDS, KS, MAXW>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes)
     switch (N) {
         case 8:
-            return stage_b ? launch_spmm<1, true, true, 8>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes)
-                           : launch_spmm<1, true, false, 8>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes);
+            return mode ? TCSL_GO(1, true, false, true, 8)
+                        : (stage_b ? TCSL_GO(1, true, true, false, 8) : TCSL_GO(1, true, false, false, 8));
         case 16:
-            return stage_b ? launch_spmm<1, false, true, 8>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes)
-                           : launch_spmm<1, false, false, 8>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes);
+            return mode ? TCSL_GO(1, false, false, true, 8)
+                        : (stage_b ? TCSL_GO(1, false, true, false, 8) : TCSL_GO(1, false, false, false, 8));
         case 32:
-            return launch_spmm<2, false, false, 4>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes);
+            return mode ? TCSL_GO(2, false, false, true, 8) : TCSL_GO(2, false, false, false, 8);
         case 64:
-            return launch_spmm<4, false, false, 4>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes);
+            return mode ? TCSL_GO(4, false, false, true, 4) : TCSL_GO(4, false, false, false, 4);
         default:
             return static_cast<int>(hipErrorInvalidValue);
     }
+#undef TCSL_GO
 }
 
 extern "C" int tcsl_launch_reduce(void* stream, void* C, const void* W, long mn, int split_k)

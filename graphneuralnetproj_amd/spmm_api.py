@@ -31,6 +31,8 @@ EXPORTED_SYMBOLS = (
     "SpMM_FreeHost",
     "SpMM_GetErrorString",
     "SpMM_SuggestSplitK",
+    "SpMM_PlanLaunch",
+    "SpMM_SplitK_API_Planned",
     "SpMM_SynthWeights",
     "SpMM_SynthActivations",
     "SpMM_CalibrationCopy",
@@ -98,6 +100,11 @@ def load_library():
     lib.SpMM_GetErrorString.argtypes = [ctypes.c_int]
     lib.SpMM_SuggestSplitK.restype = ctypes.c_int
     lib.SpMM_SuggestSplitK.argtypes = [ctypes.c_int] * 3
+    lib.SpMM_PlanLaunch.restype = ctypes.c_int
+    lib.SpMM_PlanLaunch.argtypes = [ctypes.c_int] * 4 + [_i32p] * 4 + [ctypes.POINTER(ctypes.c_double)]
+    lib.SpMM_SplitK_API_Planned.restype = ctypes.c_int
+    lib.SpMM_SplitK_API_Planned.argtypes = ([ctypes.c_void_p] * 5 + [ctypes.c_int] * 3 + [ctypes.c_void_p]
+                                            + [ctypes.c_int] * 4)
     lib.SpMM_SynthWeights.restype = None
     lib.SpMM_SynthWeights.argtypes = [_u16p, ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_int,
                                       ctypes.c_uint64]
@@ -195,6 +202,32 @@ def GenSparseMatrixBinFile(DenseMatrixFileName, M, K, NZWeightsFileName, TileOff
 
 def SpMM_SuggestSplitK(M_Global, N_Global, K_Global):
     return load_library().SpMM_SuggestSplitK(M_Global, N_Global, K_Global)
+
+
+def SpMM_PlanLaunch(M_Global, N_Global, K_Global, Split_K):
+    """The planner's launch shape for a call: dict(mode, waves, stage_b, lds_bytes, estimated_us)."""
+    vals = [ctypes.c_int() for _ in range(4)]
+    est = ctypes.c_double()
+    rc = load_library().SpMM_PlanLaunch(M_Global, N_Global, K_Global, Split_K, *[ctypes.byref(v) for v in vals],
+                                        ctypes.byref(est))
+    if rc != 0:
+        raise SpMMError("SpMM_PlanLaunch", rc)
+    return {"mode": vals[0].value, "waves": vals[1].value, "stage_b": vals[2].value, "lds_bytes": vals[3].value,
+            "estimated_us": est.value}
+
+
+def SpMM_SplitK_API_Planned(stream, Compressed_A, TileOffsets, B, C, M_Global, N_Global, K_Global,
+                            Reduction_Workspace, Split_K, Mode, Waves, StageB):
+    """SpMM_SplitK_API with a caller-chosen launch shape (tuning and tests)."""
+    lib = load_library()
+    if stream is not None and not isinstance(stream, int):
+        stream = stream.cuda_stream
+    rc = lib.SpMM_SplitK_API_Planned(ctypes.c_void_p(stream) if stream else None, _ptr(Compressed_A), _ptr(TileOffsets),
+                                     _ptr(B), _ptr(C), M_Global, N_Global, K_Global, _ptr(Reduction_Workspace),
+                                     Split_K, Mode, Waves, StageB)
+    if rc != 0:
+        raise SpMMError("SpMM_SplitK_API_Planned", rc, lib.SpMM_GetErrorString(rc).decode())
+    return rc
 
 
 def synth_weights(M, K, sparsity, row_skewed=False, seed=0):

@@ -122,11 +122,36 @@ SPMM_EXPORT void SpMM_FreeHost(void* p);
 SPMM_EXPORT const char* SpMM_GetErrorString(int code);
 
 /*
- * A Split_K that fills the 256 compute units of an MI355X for this shape; the
- * counterpart of the reference's hand-tuned per-shape table
- * (kernel_benchmark/benchmark.sh:15, huggingface_opt_convert_Phase2.py:20).
+ * The Split_K that the library's launch planner expects to be fastest for this shape
+ * on an MI355X (256 compute units); the counterpart of the reference's hand-tuned
+ * per-shape table (kernel_benchmark/benchmark.sh:15, huggingface_opt_convert_Phase2.py:20).
+ * Measured optima are built in for the OPT-30B and OPT-66B layer shapes; other shapes
+ * go through an analytic cost model.  Returns 1 for shapes the kernels do not take.
  */
 SPMM_EXPORT int SpMM_SuggestSplitK(int M_Global, int N_Global, int K_Global);
+
+/*
+ * The launch shape SpMM_SplitK_API uses for (M, N, K, Split_K):
+ *   Mode 0  the Waves waves of a workgroup take consecutive 128-row tile rows of one
+ *           split-K batch (StageB: they share the batch's activation slice in LDS);
+ *   Mode 1  the Waves waves of a workgroup split the batch of one tile row among
+ *           themselves and add their accumulators up in LDS.
+ * Any output pointer may be NULL.  EstimatedUs is the cost model's figure for the whole
+ * call.  Returns 0, or -1 for a shape the kernels do not take.  The reference has one
+ * fixed block shape (csrc/SpMM_API.cu:25-71) and nothing like this.
+ */
+SPMM_EXPORT int SpMM_PlanLaunch(int M_Global, int N_Global, int K_Global, int Split_K, int* Mode, int* Waves, int* StageB,
+                                int* LdsBytes, double* EstimatedUs);
+
+/*
+ * SpMM_SplitK_API with the launch shape given by the caller instead of the planner
+ * (for tuning a table of plans on the target machine, and for tests).  Returns
+ * hipErrorInvalidValue when the shape does not fit (Waves above 8, or 4 for N = 64;
+ * StageB with Mode 1 or N > 16; more than 160 KiB of LDS).  No counterpart in the reference.
+ */
+SPMM_EXPORT int SpMM_SplitK_API_Planned(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
+                                        void* C, int M_Global, int N_Global, int K_Global, void* Reduction_Workspace,
+                                        int Split_K, int Mode, int Waves, int StageB);
 
 /*
  * Deterministic synthetic inputs for tests and benchmarks (host memory, fp16 bit

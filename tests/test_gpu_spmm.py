@@ -267,3 +267,54 @@ def test_midsize_rows_sampled(spmm, oracle):
     C, _ = run_gpu(spmm, items, offsets, B, M, N, K, 7)
     ref = oracle.gemm_f32(A, B)
     assert_close(C, ref)
+
+
+PLANS = [
+    # (M, K, N, split_k, mode, waves, stage_b)
+    (1024, 1024, 16, 4, 0, 7, 1),    # shared slice, partial last workgroup (8 tile rows over 7 waves)
+    (1024, 1024, 16, 4, 0, 8, 1),
+    (1024, 1024, 8, 2, 0, 5, 1),
+    (1024, 1024, 16, 3, 0, 3, 0),    # fragments from global memory
+    (1024, 1024, 32, 4, 0, 4, 0),
+    (1024, 1024, 64, 2, 0, 2, 0),
+    (1024, 1024, 16, 1, 1, 8, 0),    # K split inside the workgroup, direct write of C
+    (1024, 1024, 8, 1, 1, 7, 0),     # 16 tiles over 7 waves: runs of 3, last wave gets 1... and one gets none
+    (1024, 1024, 16, 2, 1, 6, 0),
+    (1024, 1024, 32, 1, 1, 8, 0),
+    (1024, 1024, 32, 3, 1, 3, 0),
+    (1024, 1024, 64, 1, 1, 4, 0),
+    (1024, 1024, 64, 2, 1, 3, 0),
+    (256, 64 * 3, 16, 1, 1, 8, 0),   # fewer tiles than waves: five waves have nothing to do
+    (256, 64 * 70, 16, 1, 1, 1, 0),  # one wave, more than 63 tiles: the offsets window slides
+    (384, 64 * 130, 8, 1, 1, 2, 0),
+]
+
+
+@pytest.mark.parametrize("M,K,N,split_k,mode,waves,stage_b", PLANS)
+def test_explicit_launch_plans(spmm, oracle, M, K, N, split_k, mode, waves, stage_b):
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    A, B, items, offsets = make_case(spmm, M, K, N, 0.8, seed=M + K + N + 7 * mode + waves)
+    ref = oracle.gemm_f32(A, B)
+    d_items = torch.from_numpy(items.view(np.int32).copy()).to(dev)
+    d_offs = torch.from_numpy(offsets.copy()).to(dev)
+    d_B = torch.from_numpy(np.ascontiguousarray(B).view(np.int16).copy()).to(dev)
+    d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device=dev)
+    d_W = torch.full((split_k, N, M), float("nan"), dtype=torch.float16, device=dev) if split_k > 1 else None
+    print(f"[gpu case] planned M={M} N={N} K={K} split_k={split_k} mode={mode} waves={waves} stage={stage_b}", flush=True)
+    spmm.SpMM_SplitK_API_Planned(torch.cuda.current_stream(), d_items, d_offs, d_B, d_C, M, N, K, d_W, split_k, mode,
+                                 waves, stage_b)
+    torch.cuda.synchronize()
+    assert_close(d_C.cpu().numpy(), ref)
+
+
+def test_explicit_plan_rejects_what_does_not_fit(spmm):
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    z = torch.zeros(1024, dtype=torch.int32, device=dev)
+    for (N, mode, waves, stage) in [(16, 0, 9, 0), (64, 1, 5, 0), (32, 0, 2, 1), (16, 1, 4, 1), (16, 2, 4, 0), (16, 0, 0, 0)]:
+        with pytest.raises(spmm.SpMMError):
+            spmm.SpMM_SplitK_API_Planned(None, z, z, z, z, 1024, N, 1024, z, 1, mode, waves, stage)
+    # a staged slice that does not fit in LDS: 448 tiles x 16 tokens x 128 B
+    with pytest.raises(spmm.SpMMError):
+        spmm.SpMM_SplitK_API_Planned(None, z, z, z, z, 1024, 16, 28672, z, 1, 0, 4, 1)

@@ -136,7 +136,45 @@ def test_synthetic_inputs_are_deterministic_and_shaped(spmm):
     assert row_dens.std() > 0.08 and abs(row_dens.mean() - 0.2) < 0.03  # Beta(2,8): sd 0.12
 
 
+SHAPES = [(28672, 7168), (7168, 28672), (21504, 7168), (7168, 7168), (36864, 9216), (9216, 36864), (1024, 1024),
+          (128, 64), (4096, 4096), (14336, 4096), (53248, 13312), (384, 64 * 97)]
+
+
 def test_suggest_split_k(spmm):
-    for (M, K) in [(28672, 7168), (7168, 28672), (21504, 7168), (7168, 7168), (36864, 9216), (9216, 36864), (1024, 1024)]:
+    for (M, K) in SHAPES:
+        for N in (8, 16, 32, 64):
+            s = spmm.SpMM_SuggestSplitK(M, N, K)
+            assert 1 <= s <= min(32, K // 64)
+            # no batch may be empty: the last one starts inside the matrix
+            tiles = -(-(K // 64) // s)
+            assert tiles * (s - 1) < K // 64
+    assert spmm.SpMM_SuggestSplitK(1024, 24, 1024) == 1  # a token count the kernels do not take
+
+
+def test_planner_gives_runnable_plans(spmm):
+    for (M, K) in SHAPES:
+        for N in (8, 16, 32, 64):
+            for s in (1, 2, 3, 7, 8, 32):
+                if s > K // 64:
+                    continue
+                p = spmm.SpMM_PlanLaunch(M, N, K, s)
+                assert p["mode"] in (0, 1)
+                assert 1 <= p["waves"] <= (8 if N <= 32 else 4)
+                assert p["lds_bytes"] <= 160 * 1024
+                assert p["lds_bytes"] >= p["waves"] * 16384
+                if p["stage_b"]:
+                    assert p["mode"] == 0 and N <= 16
+                assert 0 < p["estimated_us"] < 1e6
+    with pytest.raises(spmm.SpMMError):
+        spmm.SpMM_PlanLaunch(1000, 16, 1024, 1)
+    with pytest.raises(spmm.SpMMError):
+        spmm.SpMM_PlanLaunch(1024, 12, 1024, 1)
+
+
+def test_planner_uses_every_compute_unit_on_the_headline_shapes(spmm):
+    # one round of workgroups, at least 200 of them, for the big OPT layers at N = 16
+    for (M, K) in [(28672, 7168), (7168, 28672), (36864, 9216), (9216, 36864)]:
         s = spmm.SpMM_SuggestSplitK(M, 16, K)
-        assert 1 <= s <= K // 64
+        p = spmm.SpMM_PlanLaunch(M, 16, K, s)
+        wgs = (M // 128) * s if p["mode"] == 1 else -(-(M // 128) // p["waves"]) * s
+        assert 200 <= wgs <= 512, (M, K, s, p)
