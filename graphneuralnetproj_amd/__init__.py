@@ -5,6 +5,7 @@ from .spmm_api import (  # noqa: F401
     SpMM_PlanLaunch,
     SpMM_SplitK_API,
     SpMM_SplitK_API_Planned,
+    SpMM_SplitK_API_RowMajor,
     SpMM_SuggestSplitK,
     SpMMError,
     build_library,

@@ -66,7 +66,7 @@ const Tuned* find_tuned(int M, int N, int K)
 
 }  // namespace
 
-bool complete_plan(int N, int K, int split_k, LaunchPlan& p)
+bool complete_plan(int N, int K, int split_k, bool row_major, LaunchPlan& p)
 {
     if (N != 8 && N != 16 && N != 32 && N != 64)
         return false;
@@ -76,6 +76,11 @@ bool complete_plan(int N, int K, int split_k, LaunchPlan& p)
     const long nkb = K / kTileCols;
     const long tiles = (nkb - 1) / split_k + 1;  // tiles of the longest batch
     long lds = p.waves * kTileLds;
+    if (row_major) {
+        if (p.stage_b)
+            return false;
+        lds += static_cast<long>(p.waves) * N * 128;  // one tile's activations per wave, being transposed
+    }
     if (p.mode == 0) {
         if (p.stage_b) {
             if (nb != 1)
@@ -141,11 +146,11 @@ double plan_cost_us(int M, int N, int K, int split_k, const LaunchPlan& p)
     return total;
 }
 
-LaunchPlan plan_launch(int M, int N, int K, int split_k, double* cost_us)
+LaunchPlan plan_launch(int M, int N, int K, int split_k, bool row_major, double* cost_us)
 {
     if (const Tuned* t = find_tuned(M, N, K)) {
         LaunchPlan p{t->mode, t->waves, t->stage_b, 0};
-        if (t->split_k == split_k && complete_plan(N, K, split_k, p)) {
+        if (t->split_k == split_k && complete_plan(N, K, split_k, row_major, p)) {
             if (cost_us)
                 *cost_us = plan_cost_us(M, N, K, split_k, p);
             return p;
@@ -157,7 +162,7 @@ LaunchPlan plan_launch(int M, int N, int K, int split_k, double* cost_us)
         for (int w = 1; w <= max_waves(N); w++)
             for (int stage = 0; stage <= (mode == 0 ? 1 : 0); stage++) {
                 LaunchPlan p{mode, w, stage, 0};
-                if (!complete_plan(N, K, split_k, p))
+                if (!complete_plan(N, K, split_k, row_major, p))
                     continue;
                 const double c = plan_cost_us(M, N, K, split_k, p);
                 if (best_cost < 0 || c < best_cost) {
@@ -174,7 +179,7 @@ int suggest_split_k(int M, int N, int K, LaunchPlan* plan)
 {
     if (const Tuned* t = find_tuned(M, N, K)) {
         LaunchPlan p{t->mode, t->waves, t->stage_b, 0};
-        if (complete_plan(N, K, t->split_k, p)) {
+        if (complete_plan(N, K, t->split_k, false, p)) {
             if (plan)
                 *plan = p;
             return t->split_k;
@@ -189,7 +194,7 @@ int suggest_split_k(int M, int N, int K, LaunchPlan* plan)
         if (s > 1 && tiles * (s - 1) >= nkb)
             continue;  // a split that leaves the last batch empty
         double c = 0.0;
-        const LaunchPlan p = plan_launch(M, N, K, static_cast<int>(s), &c);
+        const LaunchPlan p = plan_launch(M, N, K, static_cast<int>(s), false, &c);
         if (best_cost < 0 || c < best_cost - 1e-9) {
             best = static_cast<int>(s);
             best_cost = c;

@@ -15,13 +15,14 @@ struct LaunchPlan {
 };
 
 // True (and lds_bytes filled in) when the kernels can run this shape.
-bool complete_plan(int N, int K, int split_k, LaunchPlan& p);
+bool complete_plan(int N, int K, int split_k, bool row_major, LaunchPlan& p);
 
 // Estimated time in microseconds of SpMM_SplitK_API (main kernel + reduction) with this plan.
 double plan_cost_us(int M, int N, int K, int split_k, const LaunchPlan& p);
 
 // Best plan for a given Split_K; *cost_us (optional) receives its estimate.
-LaunchPlan plan_launch(int M, int N, int K, int split_k, double* cost_us);
+// row_major: B is [K][N] and C [M][N]; such calls cannot stage the activation slice.
+LaunchPlan plan_launch(int M, int N, int K, int split_k, bool row_major, double* cost_us);
 
 // Best Split_K in 1..32 (with its plan) for the shape.
 int suggest_split_k(int M, int N, int K, LaunchPlan* plan);

@@ -11,7 +11,7 @@
 
 extern "C" {
 int tcsl_launch_spmm(void* stream, const void* items, const int* offsets, const void* B, void* out, int M, int N,
-                     int K, int split_k, int mode, int waves, int stage_b, unsigned lds_bytes);
+                     int K, int split_k, int mode, int waves, int stage_b, int row_major, unsigned lds_bytes);
 int tcsl_launch_reduce(void* stream, void* C, const void* W, long mn, int split_k);
 int tcsl_launch_copy(void* stream, void* dst, const void* src, long bytes);
 void* tcsl_event_create(void);
@@ -50,34 +50,36 @@ namespace {
 
 // Plans are a pure function of the shape; the last few are remembered per thread so that a
 // decode loop cycling over a handful of layer shapes never re-runs the model.
-tcsl::LaunchPlan cached_plan(int M, int N, int K, int Split_K)
+tcsl::LaunchPlan cached_plan(int M, int N, int K, int Split_K, bool row_major)
 {
     struct Entry {
         int M, N, K, S;
+        bool row_major;
         tcsl::LaunchPlan plan;
     };
     constexpr int kEntries = 16;
     thread_local Entry cache[kEntries] = {};
     thread_local int next = 0;
     for (const Entry& e : cache)
-        if (e.M == M && e.N == N && e.K == K && e.S == Split_K)
+        if (e.M == M && e.N == N && e.K == K && e.S == Split_K && e.row_major == row_major)
             return e.plan;
-    const tcsl::LaunchPlan p = tcsl::plan_launch(M, N, K, Split_K, nullptr);
-    cache[next] = Entry{M, N, K, Split_K, p};
+    const tcsl::LaunchPlan p = tcsl::plan_launch(M, N, K, Split_K, row_major, nullptr);
+    cache[next] = Entry{M, N, K, Split_K, row_major, p};
     next = (next + 1) % kEntries;
     return p;
 }
 
 int launch_main(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* out, int M, int N,
-                int K, int Split_K, const tcsl::LaunchPlan* forced)
+                int K, int Split_K, bool row_major, const tcsl::LaunchPlan* forced)
 {
-    const tcsl::LaunchPlan p = forced ? *forced : cached_plan(M, N, K, Split_K);
+    const tcsl::LaunchPlan p = forced ? *forced : cached_plan(M, N, K, Split_K, row_major);
     return tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, out, M, N, K, Split_K, p.mode, p.waves, p.stage_b,
-                            p.lds_bytes);
+                            row_major ? 1 : 0, p.lds_bytes);
 }
 
 int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* C, int M, int N,
-                int K, void* Reduction_Workspace, int Split_K, void* ev_begin, void* ev_end, const tcsl::LaunchPlan* forced);
+                int K, void* Reduction_Workspace, int Split_K, void* ev_begin, void* ev_end, bool row_major,
+                const tcsl::LaunchPlan* forced);
 }
 
 extern "C" int SpMM_SplitK_API(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets,
@@ -85,18 +87,27 @@ extern "C" int SpMM_SplitK_API(void* stream, const void* A, const void* Compress
 {
     (void)A;
     return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, nullptr,
-                       nullptr, nullptr);
+                       nullptr, false, nullptr);
+}
+
+extern "C" int SpMM_SplitK_API_RowMajor(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets,
+                                        const void* B, void* C, int M, int N, int K, void* Reduction_Workspace,
+                                        int Split_K)
+{
+    (void)A;
+    return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, nullptr,
+                       nullptr, true, nullptr);
 }
 
 extern "C" int SpMM_SplitK_API_Planned(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
                                        void* C, int M, int N, int K, void* Reduction_Workspace, int Split_K, int Mode,
-                                       int Waves, int StageB)
+                                       int Waves, int StageB, int RowMajor)
 {
     tcsl::LaunchPlan p{Mode, Waves, StageB, 0};
-    if (!tcsl::complete_plan(N, K > 0 ? K : 64, Split_K, p))
+    if (!tcsl::complete_plan(N, K > 0 ? K : 64, Split_K, RowMajor != 0, p))
         return tcsl_error_invalid_value();
     return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, nullptr,
-                       nullptr, &p);
+                       nullptr, RowMajor != 0, &p);
 }
 
 extern "C" int SpMM_PlanLaunch(int M, int N, int K, int Split_K, int* Mode, int* Waves, int* StageB, int* LdsBytes,
@@ -106,7 +117,7 @@ extern "C" int SpMM_PlanLaunch(int M, int N, int K, int Split_K, int* Mode, int*
         K % tcsl::kTileCols != 0 || Split_K < 1)
         return -1;
     double cost = 0.0;
-    const tcsl::LaunchPlan p = tcsl::plan_launch(M, N, K, Split_K, &cost);
+    const tcsl::LaunchPlan p = tcsl::plan_launch(M, N, K, Split_K, false, &cost);
     if (Mode)
         *Mode = p.mode;
     if (Waves)
@@ -126,7 +137,7 @@ extern "C" int SpMM_SplitK_API_Events(void* stream, const void* A, const void* C
 {
     (void)A;
     return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, KernelBegin,
-                       KernelEnd, nullptr);
+                       KernelEnd, false, nullptr);
 }
 
 extern "C" int SpMM_SplitK_Partials(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
@@ -139,7 +150,7 @@ extern "C" int SpMM_SplitK_Partials(void* stream, const void* Compressed_A, cons
         return tcsl_error_invalid_value();
     if (!Compressed_A || !TileOffsets || !B || !Partials)
         return tcsl_error_invalid_value();
-    return launch_main(stream, Compressed_A, TileOffsets, B, Partials, M, N, K, Split_K, nullptr);
+    return launch_main(stream, Compressed_A, TileOffsets, B, Partials, M, N, K, Split_K, false, nullptr);
 }
 
 extern "C" void* SpMM_EventCreate(void)
@@ -165,7 +176,7 @@ extern "C" float SpMM_EventElapsedMs(void* start, void* stop)
 namespace {
 
 int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* C, int M, int N,
-                int K, void* Reduction_Workspace, int Split_K, void* ev_begin, void* ev_end,
+                int K, void* Reduction_Workspace, int Split_K, void* ev_begin, void* ev_end, bool row_major,
                 const tcsl::LaunchPlan* forced)
 {
     if (N != 8 && N != 16 && N != 32 && N != 64) {
@@ -191,7 +202,7 @@ int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, 
     if (ev_begin && (rc = tcsl_event_record(ev_begin, stream)) != 0)
         return rc;
     rc = launch_main(stream, Compressed_A, TileOffsets, B, Split_K == 1 ? C : Reduction_Workspace, M, N, K, Split_K,
-                     forced);
+                     row_major, forced);
     if (rc != 0)
         return rc;
     if (ev_end && (rc = tcsl_event_record(ev_end, stream)) != 0)

@@ -97,6 +97,14 @@ __device__ __forceinline__ half8 load_activations(const _Float16* p)
     return r;
 }
 
+// 16 bytes per lane at base + voff (uniform 64-bit base, per-lane 32-bit byte offset)
+__device__ __forceinline__ half8 load_activations_at(const _Float16* base, uint32_t voff)
+{
+    half8 r;
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r) : "v"(voff), "s"(base));
+    return r;
+}
+
 // Wait until at most N vector-memory loads are outstanding (they complete in order).
 template<int N>
 __device__ __forceinline__ void wait_loads()
@@ -152,11 +160,12 @@ __device__ __forceinline__ void clear_tile(uint8_t* tile, int lane)
 
 // blockDim.x = W * 64.  Wave w of workgroup g owns tile row (g % groups) * W + w of batch
 // g / groups, groups = ceil(tile rows / W).  NB = number of 16-token column blocks;
-// HALF = N is 8 (the upper eight columns of the single block are computed on duplicates
+// ROWMAJ = B is [K][N] and the output [M][N].  HALF = N is 8 (the upper eight columns of the single block are computed on duplicates
 // and dropped); BLDS = the batch's activation slice is staged in LDS; MAXW bounds W and
 // with it the registers a wave may use.
-// Dynamic LDS: W tiles of 16 KiB, then (BLDS) tiles_per_batch * tokens * 128 bytes.
-template<int NB, bool HALF, bool BLDS, bool KSPLIT, int MAXW>
+// Dynamic LDS: W tiles of 16 KiB, then tokens * 128 bytes times tiles_per_batch (BLDS) or times W
+// (ROWMAJ); with KSPLIT at least 8 * W * NB KiB in all (the waves' accumulators meet there).
+template<int NB, bool HALF, bool BLDS, bool KSPLIT, bool ROWMAJ, int MAXW>
 __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __restrict__ items,
                                                                 const int* __restrict__ offsets,
                                                                 const _Float16* __restrict__ B,
@@ -166,11 +175,15 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int VPL = kVecPerLane;
     constexpr int D = kRing;
-    constexpr int L = VPL + (BLDS ? 0 : 2 * NB);  // loads per issue: word loads (+ activation loads)
+    constexpr int NTOK = HALF ? 8 : NB * 16;      // tokens
+    // activation loads per issue: two fragments per column block, or (ROWMAJ) the tile's
+    // 64 x N block as 1 KiB pieces
+    constexpr int BL = BLDS ? 0 : (ROWMAJ ? NTOK / 8 : 2 * NB);
+    constexpr int L = VPL + BL;                   // loads per issue: word loads (+ activation loads)
     constexpr int kSeg = VPL * kWave;             // vectors per segment
-    constexpr int NTOK = HALF ? 8 : NB * 16;      // tokens in the staged slice
 
     static_assert(!(KSPLIT && BLDS), "a workgroup that splits K shares no activation slice");
+    static_assert(!(ROWMAJ && BLDS), "row-major activations are not staged");
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // uniform, and known to be
     const int W = blockDim.x / kWave;
@@ -196,7 +209,10 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
     }
     const int ntile = kb1 - kb0;  // tiles of this wave
     uint8_t* const tile = lds + wave * kTileBytes;
-    uint8_t* const bslice = lds + W * kTileBytes;  // [tile][token][8 granules of 16 B at position g ^ (token & 7)]
+    // Activations in LDS, per tile [token][8 granules of 16 B at position g ^ (token & 7)]: the
+    // batch's slice, staged once and shared (BLDS), or (ROWMAJ) a one-tile buffer per wave in
+    // which the tile's k-major block is turned into token-major MFMA operands.
+    uint8_t* const bslice = lds + W * kTileBytes + (ROWMAJ ? wave * (NTOK * 128) : 0);
 
     // Offsets window: lane l holds toff[wbase + l]; toff[i] = first vector of tile i,
     // toff[ntile] = end.  Issued first so its latency overlaps the staging below.
@@ -258,7 +274,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
         int tok = c * 16 + l15;
         if (HALF)
             tok &= 7;
-        bptr[c] = B + (size_t)tok * K + (size_t)kb0 * kTileCols + q * 8;
+        bptr[c] = ROWMAJ ? B : B + (size_t)tok * K + (size_t)kb0 * kTileCols + q * 8;
 #pragma unroll
         for (int s = 0; s < 2; s++)
             b_off[c][s] = tok * 128 + (((s * 4 + q) ^ (tok & 7)) << 4);
@@ -300,7 +316,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
     };
 
     u32x4 regs[D][VPL];
-    half8 bfrag[D][NB][2];  // only used when the activations come from global memory
+    half8 bfrag[D][BL > 0 ? BL : 1];  // only used when the activations come from global memory
     Seg held[D];
 
     // Always exactly L loads, whatever the segment holds, so the wait counts are static.
@@ -322,11 +338,19 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
         });
         if (!BLDS) {
             const int bt = live ? s.tile : ntile - 1;
+            if (ROWMAJ) {
+                // B[k][n]: the tile's 64 x N block is contiguous; piece h = bytes [1024 h, 1024 h + 1024)
+                const _Float16* blk = B + (size_t)(kb0 + bt) * (kTileCols * NTOK);
 #pragma unroll
-            for (int cb = 0; cb < NB; cb++)
+                for (int h = 0; h < BL; h++)
+                    bfrag[slot][h] = load_activations_at(blk + h * 512, lane * 16);
+            } else {
 #pragma unroll
-                for (int k = 0; k < 2; k++)
-                    bfrag[slot][cb][k] = load_activations(bptr[cb] + bt * kTileCols + k * 32);
+                for (int cb = 0; cb < NB; cb++)
+#pragma unroll
+                    for (int k = 0; k < 2; k++)
+                        bfrag[slot][cb * 2 + k] = load_activations(bptr[cb] + bt * kTileCols + k * 32);
+            }
         }
     };
 
@@ -339,10 +363,8 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
         static_for<VPL>([&](auto uc) { pin(regs[slot][decltype(uc)::value]); });
         if (!BLDS) {
 #pragma unroll
-            for (int cb = 0; cb < NB; cb++)
-#pragma unroll
-                for (int k = 0; k < 2; k++)
-                    settle(bfrag[slot][cb][k]);
+            for (int h = 0; h < BL; h++)
+                settle(bfrag[slot][h]);
         }
     };
 
@@ -365,8 +387,21 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
         if (!s.last)
             return;  // more segments of this tile follow
         half8 bf[NB][2];
-        if (BLDS) {
-            const uint8_t* bt = bslice + (size_t)s.tile * (NTOK * 128);
+        if (BLDS || ROWMAJ) {
+            const uint8_t* bt = bslice + (BLDS ? (size_t)s.tile * (NTOK * 128) : 0);
+            if (ROWMAJ) {
+                // lane l of piece h holds tokens n0 .. n0+7 of row k, (k, n0) = divmod(512 h + 8 l, N);
+                // element (k, n) goes to byte n*128 + (((k >> 3) ^ (n & 7)) << 4) + 2*(k & 7), n & 7 = j
+#pragma unroll
+                for (int h = 0; h < BL; h++) {
+                    const int e0 = h * 512 + lane * 8;
+                    const int k = e0 / NTOK, n0 = e0 % NTOK;
+                    const int base = n0 * 128 + (k & 7) * 2, g0 = (k >> 3) << 4;
+#pragma unroll
+                    for (int j = 0; j < 8; j++)
+                        *reinterpret_cast<_Float16*>(bslice + ((g0 ^ (j << 4)) + base) + j * 128) = bfrag[slot][h][j];
+                }
+            }
 #pragma unroll
             for (int cb = 0; cb < NB; cb++)
 #pragma unroll
@@ -377,7 +412,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
             for (int cb = 0; cb < NB; cb++)
 #pragma unroll
                 for (int k = 0; k < 2; k++)
-                    bf[cb][k] = bfrag[slot][cb][k];
+                    bf[cb][k] = bfrag[slot][cb * 2 + k];
         }
         // read the dense tile back and multiply; all reads of a pass are issued before its MFMAs
         constexpr int kPasses = NB == 1 ? 1 : 2;
@@ -449,7 +484,9 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
     // c*16 + l15; the output keeps one contiguous M vector per token.  The block goes through
     // the wave's LDS tile as [token][128 rows] (token stride padded to 272 B) so that the
     // global stores are 16 bytes per lane with 16 lanes covering a token's 256 bytes.
-    _Float16* oslab = out + (size_t)batch * M * N + (size_t)rt * kTileRows;
+    // column-major: C[token][M], this wave's 128 rows start at rt * 128 of every token's vector;
+    // row-major: C[M][N], this wave's rows are one contiguous block of 128 * N values
+    _Float16* oslab = out + (size_t)batch * M * N + (size_t)rt * kTileRows * (ROWMAJ ? NTOK : 1);
     if (KSPLIT) {
         // Sum the W waves' accumulators through LDS, in wave order.  Layout: [row block r]
         // [source wave][column block c][lane] x 16 bytes; wave w then owns row blocks w, w + W, ...
@@ -476,10 +513,38 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
 #pragma unroll
                 for (int i = 0; i < 4; i++)
                     h[i] = static_cast<_Float16>(sum[i]);
-                // rows r*16 + 4*q .. +3 of token c*16 + l15: the four q-lanes of a token cover 32 bytes
-                if (!(HALF && l15 >= 8))
-                    *reinterpret_cast<half4*>(oslab + (size_t)(c * 16 + l15) * M + r * 16 + q * 4) = h;
+                // rows r*16 + 4*q .. +3 of token c*16 + l15
+                if (!(HALF && l15 >= 8)) {
+                    if (ROWMAJ) {
+#pragma unroll
+                        for (int i = 0; i < 4; i++)  // the 16 tokens of a row are adjacent
+                            oslab[(r * 16 + q * 4 + i) * NTOK + c * 16 + l15] = h[i];
+                    } else {  // the four q-lanes of a token cover 32 bytes
+                        *reinterpret_cast<half4*>(oslab + (size_t)(c * 16 + l15) * M + r * 16 + q * 4) = h;
+                    }
+                }
             }
+        }
+        return;
+    }
+    if (ROWMAJ) {
+        // the wave's 128 x N block through its LDS tile in memory order, then 16 bytes per lane
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the last tile's clearing writes
+        if (!(HALF && l15 >= 8)) {
+#pragma unroll
+            for (int c = 0; c < NB; c++)
+#pragma unroll
+                for (int r = 0; r < 8; r++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        *reinterpret_cast<_Float16*>(tile + ((r * 16 + q * 4 + i) * NTOK + c * 16 + l15) * 2) =
+                            static_cast<_Float16>(acc[c][r][i]);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // other lanes read what this lane wrote
+#pragma unroll
+        for (int i = 0; i < kTileRows * NTOK * 2 / (kWave * 16); i++) {
+            const half8 v = *reinterpret_cast<const half8*>(tile + (i * kWave + lane) * 16);
+            *reinterpret_cast<half8*>(oslab + (i * kWave + lane) * 8) = v;
         }
         return;
     }
@@ -557,13 +622,13 @@ __global__ __launch_bounds__(256) void tcsl_copy_kernel(u32x4* __restrict__ dst,
         dst[i] = src[i];
 }
 
-template<int NB, bool HALF, bool BLDS, bool KSPLIT, int MAXW>
+template<int NB, bool HALF, bool BLDS, bool KSPLIT, bool ROWMAJ, int MAXW>
 int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const void* B, void* out, int M, int N,
                 int K, int split_k, int waves, unsigned lds_bytes)
 {
     if (waves < 1 || waves > MAXW || lds_bytes > kMaxLdsBytes)
         return static_cast<int>(hipErrorInvalidValue);
-    auto kernel = tcsl_spmm_kernel<NB, HALF, BLDS, KSPLIT, MAXW>;
+    auto kernel = tcsl_spmm_kernel<NB, HALF, BLDS, KSPLIT, ROWMAJ, MAXW>;
     // more than 64 KiB of dynamic LDS has to be allowed once per kernel (per device, re-armed lazily)
     static std::atomic<int> armed_device{-1};
     int dev = 0;
@@ -595,31 +660,35 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
 //         stage_b != 0 and N <= 16, share the batch's activation slice in LDS);
 // mode 1: the W waves of a workgroup split the batch of one tile row among themselves and
 //         add their results up in LDS (stage_b must be 0).
-// waves = 1..8 for N <= 16, 1..4 above; lds_bytes = what the mode needs (the host plans it).
+// row_major: B is [K][N] and the output [M][N] instead of [N][K] and [N][M] (stage_b must be 0).
+// waves = 1..8 for N <= 32, 1..4 for N = 64; lds_bytes = what the shape needs (the host plans it).
 extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offsets, const void* B, void* out, int M,
-                                int N, int K, int split_k, int mode, int waves, int stage_b, unsigned lds_bytes)
+                                int N, int K, int split_k, int mode, int waves, int stage_b, int row_major,
+                                unsigned lds_bytes)
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (mode != 0 && mode != 1)
         return static_cast<int>(hipErrorInvalidValue);
-    if (mode == 1 && stage_b)
+    if (stage_b && (mode == 1 || row_major || N > 16))
         return static_cast<int>(hipErrorInvalidValue);
-#define TCSL_GO(NB, HALF, BLDS, KS, MAXW) \
-    launch_spmm<NB, HALF, BLDS, KS, MAXW>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes)
+#define TCSL_GO(NB, HALF, BLDS, KS, RM, MAXW) \
+    launch_spmm<NB, HALF, BLDS, KS, RM, MAXW>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes)
+#define TCSL_PICK(NB, HALF, MAXW)                                                                     \
+    (row_major ? (mode ? TCSL_GO(NB, HALF, false, true, true, MAXW) : TCSL_GO(NB, HALF, false, false, true, MAXW)) \
+               : (mode ? TCSL_GO(NB, HALF, false, true, false, MAXW) : TCSL_GO(NB, HALF, false, false, false, MAXW)))
     switch (N) {
         case 8:
-            return mode ? TCSL_GO(1, true, false, true, 8)
-                        : (stage_b ? TCSL_GO(1, true, true, false, 8) : TCSL_GO(1, true, false, false, 8));
+            return stage_b ? TCSL_GO(1, true, true, false, false, 8) : TCSL_PICK(1, true, 8);
         case 16:
-            return mode ? TCSL_GO(1, false, false, true, 8)
-                        : (stage_b ? TCSL_GO(1, false, true, false, 8) : TCSL_GO(1, false, false, false, 8));
+            return stage_b ? TCSL_GO(1, false, true, false, false, 8) : TCSL_PICK(1, false, 8);
         case 32:
-            return mode ? TCSL_GO(2, false, false, true, 8) : TCSL_GO(2, false, false, false, 8);
+            return TCSL_PICK(2, false, 8);
         case 64:
-            return mode ? TCSL_GO(4, false, false, true, 4) : TCSL_GO(4, false, false, false, 4);
+            return TCSL_PICK(4, false, 4);
         default:
             return static_cast<int>(hipErrorInvalidValue);
     }
+#undef TCSL_PICK
 #undef TCSL_GO
 }
 

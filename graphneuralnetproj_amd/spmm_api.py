@@ -33,6 +33,7 @@ EXPORTED_SYMBOLS = (
     "SpMM_SuggestSplitK",
     "SpMM_PlanLaunch",
     "SpMM_SplitK_API_Planned",
+    "SpMM_SplitK_API_RowMajor",
     "SpMM_SynthWeights",
     "SpMM_SynthActivations",
     "SpMM_CalibrationCopy",
@@ -104,7 +105,9 @@ def load_library():
     lib.SpMM_PlanLaunch.argtypes = [ctypes.c_int] * 4 + [_i32p] * 4 + [ctypes.POINTER(ctypes.c_double)]
     lib.SpMM_SplitK_API_Planned.restype = ctypes.c_int
     lib.SpMM_SplitK_API_Planned.argtypes = ([ctypes.c_void_p] * 5 + [ctypes.c_int] * 3 + [ctypes.c_void_p]
-                                            + [ctypes.c_int] * 4)
+                                            + [ctypes.c_int] * 5)
+    lib.SpMM_SplitK_API_RowMajor.restype = ctypes.c_int
+    lib.SpMM_SplitK_API_RowMajor.argtypes = lib.SpMM_SplitK_API.argtypes
     lib.SpMM_SynthWeights.restype = None
     lib.SpMM_SynthWeights.argtypes = [_u16p, ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_int,
                                       ctypes.c_uint64]
@@ -191,6 +194,20 @@ def SpMM_SplitK_API(stream, A, Compressed_A, TileOffsets, B, C, M_Global, N_Glob
     return rc
 
 
+def SpMM_SplitK_API_RowMajor(stream, A, Compressed_A, TileOffsets, B, C, M_Global, N_Global, K_Global,
+                             Reduction_Workspace, Split_K):
+    """SpMM_SplitK_API for row-major B (K x N) and C (M x N)."""
+    lib = load_library()
+    if stream is not None and not isinstance(stream, int):
+        stream = stream.cuda_stream
+    rc = lib.SpMM_SplitK_API_RowMajor(ctypes.c_void_p(stream) if stream else None, _ptr(A), _ptr(Compressed_A),
+                                      _ptr(TileOffsets), _ptr(B), _ptr(C), M_Global, N_Global, K_Global,
+                                      _ptr(Reduction_Workspace), Split_K)
+    if rc != 0:
+        raise SpMMError("SpMM_SplitK_API_RowMajor", rc, lib.SpMM_GetErrorString(rc).decode())
+    return rc
+
+
 def GenSparseMatrixBinFile(DenseMatrixFileName, M, K, NZWeightsFileName, TileOffsetsFileName, OutputSizesFileName):
     lib = load_library()
     rc = lib.GenSparseMatrixBinFile(DenseMatrixFileName.encode(), M, K, NZWeightsFileName.encode(),
@@ -217,14 +234,14 @@ def SpMM_PlanLaunch(M_Global, N_Global, K_Global, Split_K):
 
 
 def SpMM_SplitK_API_Planned(stream, Compressed_A, TileOffsets, B, C, M_Global, N_Global, K_Global,
-                            Reduction_Workspace, Split_K, Mode, Waves, StageB):
+                            Reduction_Workspace, Split_K, Mode, Waves, StageB, RowMajor=0):
     """SpMM_SplitK_API with a caller-chosen launch shape (tuning and tests)."""
     lib = load_library()
     if stream is not None and not isinstance(stream, int):
         stream = stream.cuda_stream
     rc = lib.SpMM_SplitK_API_Planned(ctypes.c_void_p(stream) if stream else None, _ptr(Compressed_A), _ptr(TileOffsets),
                                      _ptr(B), _ptr(C), M_Global, N_Global, K_Global, _ptr(Reduction_Workspace),
-                                     Split_K, Mode, Waves, StageB)
+                                     Split_K, Mode, Waves, StageB, RowMajor)
     if rc != 0:
         raise SpMMError("SpMM_SplitK_API_Planned", rc, lib.SpMM_GetErrorString(rc).decode())
     return rc

@@ -75,6 +75,19 @@ SPMM_EXPORT int SpMM_SplitK_API(void* stream, const void* A, const void* Compres
                     void* C, int M_Global, int N_Global, int K_Global, void* Reduction_Workspace, int Split_K);
 
 /*
+ * SpMM_SplitK_API for row-major operands: B[k*N + n] (K x N) and C[m*N + n] (M x N), with
+ * the split-K slabs in the same M x N layout.  This is the convention of this checkout's
+ * kernel (csrc/SpMM_Kernel.cuh:372-374 for B, :731-734 for the output; its benchmark passes a
+ * transposed B and transposes C back, kernel_benchmark/spmm_test.cu:137-141,474,569-576),
+ * whereas SpMM_SplitK_API keeps the column-major one of the original interface and of the
+ * FasterTransformer caller.  Same arguments, checks and return codes.  The activation
+ * block of every tile is turned token-major inside the kernel, which costs a few percent.
+ */
+SPMM_EXPORT int SpMM_SplitK_API_RowMajor(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets,
+                                         const void* B, void* C, int M_Global, int N_Global, int K_Global,
+                                         void* Reduction_Workspace, int Split_K);
+
+/*
  * SpMM_SplitK_API with two hipEvent_t recorded on `stream` immediately before and
  * after the main kernel (the split-K reduction, if any, follows KernelEnd), so a
  * benchmark can time that kernel alone inside its own loop.  Either event may be
@@ -147,11 +160,12 @@ SPMM_EXPORT int SpMM_PlanLaunch(int M_Global, int N_Global, int K_Global, int Sp
  * SpMM_SplitK_API with the launch shape given by the caller instead of the planner
  * (for tuning a table of plans on the target machine, and for tests).  Returns
  * hipErrorInvalidValue when the shape does not fit (Waves above 8, or 4 for N = 64;
- * StageB with Mode 1 or N > 16; more than 160 KiB of LDS).  No counterpart in the reference.
+ * StageB with Mode 1, N > 16 or RowMajor; more than 160 KiB of LDS).  RowMajor != 0 selects
+ * the operand layout of SpMM_SplitK_API_RowMajor.  No counterpart in the reference.
  */
 SPMM_EXPORT int SpMM_SplitK_API_Planned(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
                                         void* C, int M_Global, int N_Global, int K_Global, void* Reduction_Workspace,
-                                        int Split_K, int Mode, int Waves, int StageB);
+                                        int Split_K, int Mode, int Waves, int StageB, int RowMajor);
 
 /*
  * Deterministic synthetic inputs for tests and benchmarks (host memory, fp16 bit

@@ -315,6 +315,66 @@ def test_explicit_plan_rejects_what_does_not_fit(spmm):
     for (N, mode, waves, stage) in [(16, 0, 9, 0), (64, 1, 5, 0), (32, 0, 2, 1), (16, 1, 4, 1), (16, 2, 4, 0), (16, 0, 0, 0)]:
         with pytest.raises(spmm.SpMMError):
             spmm.SpMM_SplitK_API_Planned(None, z, z, z, z, 1024, N, 1024, z, 1, mode, waves, stage)
+    with pytest.raises(spmm.SpMMError):  # row-major operands cannot use the staged slice
+        spmm.SpMM_SplitK_API_Planned(None, z, z, z, z, 1024, 16, 1024, z, 1, 0, 4, 1, 1)
     # a staged slice that does not fit in LDS: 448 tiles x 16 tokens x 128 B
     with pytest.raises(spmm.SpMMError):
         spmm.SpMM_SplitK_API_Planned(None, z, z, z, z, 1024, 16, 28672, z, 1, 0, 4, 1)
+
+
+def _row_major_case(spmm, oracle, M, K, N, split_k, plan=None, sparsity=0.8):
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    A, B, items, offsets = make_case(spmm, M, K, N, sparsity, seed=3 * M + K + N + split_k)
+    ref = oracle.gemm_f32(A, B)  # N x M
+    d_items = torch.from_numpy(items.view(np.int32).copy()).to(dev)
+    d_offs = torch.from_numpy(offsets.copy()).to(dev)
+    Bt = np.ascontiguousarray(B.T)  # K x N
+    d_B = torch.from_numpy(Bt.view(np.int16).copy()).to(dev)
+    d_C = torch.full((M, N), float("nan"), dtype=torch.float16, device=dev)
+    d_W = torch.full((split_k, M, N), float("nan"), dtype=torch.float16, device=dev) if split_k > 1 else None
+    print(f"[gpu case] row-major M={M} N={N} K={K} split_k={split_k} plan={plan}", flush=True)
+    if plan is None:
+        spmm.SpMM_SplitK_API_RowMajor(torch.cuda.current_stream(), None, d_items, d_offs, d_B, d_C, M, N, K, d_W, split_k)
+    else:
+        spmm.SpMM_SplitK_API_Planned(torch.cuda.current_stream(), d_items, d_offs, d_B, d_C, M, N, K, d_W, split_k,
+                                     plan[0], plan[1], 0, 1)
+    torch.cuda.synchronize()
+    assert_close(d_C.cpu().numpy().T, ref)
+
+
+@pytest.mark.parametrize("N", [8, 16, 32, 64])
+@pytest.mark.parametrize("split_k", [1, 3])
+def test_row_major_entry(spmm, oracle, N, split_k):
+    _row_major_case(spmm, oracle, 512, 1024, N, split_k)
+
+
+@pytest.mark.parametrize("M,K,N,split_k,mode,waves", [
+    (1024, 1024, 16, 4, 0, 7), (1024, 1024, 8, 2, 0, 3), (1024, 1024, 32, 2, 0, 8), (1024, 1024, 64, 2, 0, 4),
+    (1024, 1024, 16, 1, 1, 8), (1024, 1024, 8, 1, 1, 5), (1024, 1024, 32, 1, 1, 6), (1024, 1024, 64, 1, 1, 4),
+    (256, 64 * 70, 16, 1, 0, 1), (128, 64, 16, 1, 1, 8),
+])
+def test_row_major_launch_shapes(spmm, oracle, M, K, N, split_k, mode, waves):
+    _row_major_case(spmm, oracle, M, K, N, split_k, plan=(mode, waves))
+
+
+def test_row_major_layout_probe(spmm, oracle):
+    """One-hot activations: C[:, n] must be column k_n of A, exactly, in M x N order."""
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    M, K, N = 256, 256, 16
+    A = spmm.synth_weights(M, K, 0.5, False, seed=77)
+    items, offsets = spmm.InitSparseMatrixA_API(A)
+    ks = [(17 * n + 3) % K for n in range(N)]
+    Bt = np.zeros((K, N), dtype=np.float16)
+    for n, k in enumerate(ks):
+        Bt[k, n] = 1.0
+    d_items = torch.from_numpy(items.view(np.int32).copy()).to(dev)
+    d_offs = torch.from_numpy(offsets.copy()).to(dev)
+    d_B = torch.from_numpy(Bt.view(np.int16).copy()).to(dev)
+    d_C = torch.full((M, N), float("nan"), dtype=torch.float16, device=dev)
+    spmm.SpMM_SplitK_API_RowMajor(None, None, d_items, d_offs, d_B, d_C, M, N, K, None, 1)
+    torch.cuda.synchronize()
+    C = d_C.cpu().numpy()
+    for n, k in enumerate(ks):
+        assert np.array_equal(C[:, n], A[:, k])
