@@ -6,6 +6,8 @@ from .spmm_api import (  # noqa: F401
     SpMM_SplitK_API,
     SpMM_SplitK_API_Planned,
     SpMM_SplitK_API_RowMajor,
+    SpMM_SplitK_API_Strided,
+    SPMM_FLAG_RELU,
     SpMM_SuggestSplitK,
     SpMMError,
     build_library,

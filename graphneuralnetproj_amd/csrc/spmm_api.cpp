@@ -11,8 +11,9 @@
 
 extern "C" {
 int tcsl_launch_spmm(void* stream, const void* items, const int* offsets, const void* B, void* out, int M, int N,
-                     int K, int split_k, int mode, int waves, int stage_b, int row_major, unsigned lds_bytes);
-int tcsl_launch_reduce(void* stream, void* C, const void* W, long mn, int split_k);
+                     int K, int split_k, int mode, int waves, int stage_b, int row_major, unsigned lds_bytes, int ldb,
+                     int ldo, int relu);
+int tcsl_launch_reduce(void* stream, void* C, const void* W, long rows, long vectors, long ldc, int split_k, int relu);
 int tcsl_launch_copy(void* stream, void* dst, const void* src, long bytes);
 void* tcsl_event_create(void);
 void tcsl_event_destroy(void* e);
@@ -69,25 +70,34 @@ tcsl::LaunchPlan cached_plan(int M, int N, int K, int Split_K, bool row_major)
     return p;
 }
 
+// What varies between the entry points that end in the same two launches.
+struct CallOptions {
+    bool row_major = false;   // B is [K][N], C and the slabs [M][N]
+    long ldb = 0;             // elements between two tokens' vectors in B (0 = K); column-major only
+    long ldc = 0;             // the same for C (0 = M)
+    bool relu = false;        // clamp C at zero
+    void* ev_begin = nullptr; // events recorded around the main kernel
+    void* ev_end = nullptr;
+    const tcsl::LaunchPlan* forced = nullptr;
+};
+
 int launch_main(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* out, int M, int N,
-                int K, int Split_K, bool row_major, const tcsl::LaunchPlan* forced)
+                int K, int Split_K, const CallOptions& o, int ldb, int ldo, bool relu)
 {
-    const tcsl::LaunchPlan p = forced ? *forced : cached_plan(M, N, K, Split_K, row_major);
+    const tcsl::LaunchPlan p = o.forced ? *o.forced : cached_plan(M, N, K, Split_K, o.row_major);
     return tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, out, M, N, K, Split_K, p.mode, p.waves, p.stage_b,
-                            row_major ? 1 : 0, p.lds_bytes);
+                            o.row_major ? 1 : 0, p.lds_bytes, ldb, ldo, relu ? 1 : 0);
 }
 
 int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* C, int M, int N,
-                int K, void* Reduction_Workspace, int Split_K, void* ev_begin, void* ev_end, bool row_major,
-                const tcsl::LaunchPlan* forced);
-}
+                int K, void* Reduction_Workspace, int Split_K, const CallOptions& o);
+}  // namespace
 
 extern "C" int SpMM_SplitK_API(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets,
                                const void* B, void* C, int M, int N, int K, void* Reduction_Workspace, int Split_K)
 {
     (void)A;
-    return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, nullptr,
-                       nullptr, false, nullptr);
+    return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, CallOptions{});
 }
 
 extern "C" int SpMM_SplitK_API_RowMajor(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets,
@@ -95,8 +105,23 @@ extern "C" int SpMM_SplitK_API_RowMajor(void* stream, const void* A, const void*
                                         int Split_K)
 {
     (void)A;
-    return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, nullptr,
-                       nullptr, true, nullptr);
+    CallOptions o;
+    o.row_major = true;
+    return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, o);
+}
+
+extern "C" int SpMM_SplitK_API_Strided(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
+                                       long ldb, void* C, long ldc, int M, int N, int K, void* Reduction_Workspace,
+                                       int Split_K, int Flags)
+{
+    if (ldb < K || ldc < M || ldb % 8 != 0 || ldc % 8 != 0 || ldb > 0x7fffffffL || ldc > 0x7fffffffL ||
+        (Flags & ~SPMM_FLAG_RELU) != 0)
+        return tcsl_error_invalid_value();
+    CallOptions o;
+    o.ldb = ldb;
+    o.ldc = ldc;
+    o.relu = (Flags & SPMM_FLAG_RELU) != 0;
+    return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, o);
 }
 
 extern "C" int SpMM_SplitK_API_Planned(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
@@ -106,8 +131,10 @@ extern "C" int SpMM_SplitK_API_Planned(void* stream, const void* Compressed_A, c
     tcsl::LaunchPlan p{Mode, Waves, StageB, 0};
     if (!tcsl::complete_plan(N, K > 0 ? K : 64, Split_K, RowMajor != 0, p))
         return tcsl_error_invalid_value();
-    return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, nullptr,
-                       nullptr, RowMajor != 0, &p);
+    CallOptions o;
+    o.row_major = RowMajor != 0;
+    o.forced = &p;
+    return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, o);
 }
 
 extern "C" int SpMM_PlanLaunch(int M, int N, int K, int Split_K, int* Mode, int* Waves, int* StageB, int* LdsBytes,
@@ -136,8 +163,10 @@ extern "C" int SpMM_SplitK_API_Events(void* stream, const void* A, const void* C
                                       int Split_K, void* KernelBegin, void* KernelEnd)
 {
     (void)A;
-    return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, KernelBegin,
-                       KernelEnd, false, nullptr);
+    CallOptions o;
+    o.ev_begin = KernelBegin;
+    o.ev_end = KernelEnd;
+    return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, o);
 }
 
 extern "C" int SpMM_SplitK_Partials(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
@@ -150,7 +179,7 @@ extern "C" int SpMM_SplitK_Partials(void* stream, const void* Compressed_A, cons
         return tcsl_error_invalid_value();
     if (!Compressed_A || !TileOffsets || !B || !Partials)
         return tcsl_error_invalid_value();
-    return launch_main(stream, Compressed_A, TileOffsets, B, Partials, M, N, K, Split_K, false, nullptr);
+    return launch_main(stream, Compressed_A, TileOffsets, B, Partials, M, N, K, Split_K, CallOptions{}, K, M, false);
 }
 
 extern "C" void* SpMM_EventCreate(void)
@@ -176,8 +205,7 @@ extern "C" float SpMM_EventElapsedMs(void* start, void* stop)
 namespace {
 
 int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* C, int M, int N,
-                int K, void* Reduction_Workspace, int Split_K, void* ev_begin, void* ev_end, bool row_major,
-                const tcsl::LaunchPlan* forced)
+                int K, void* Reduction_Workspace, int Split_K, const CallOptions& o)
 {
     if (N != 8 && N != 16 && N != 32 && N != 64) {
         std::printf("MM_Sparse_API Error: Unsupported N dimension %d!\n", N);
@@ -197,19 +225,26 @@ int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, 
         std::fprintf(stderr, "SpMM_SplitK_API: Split_K=%d too large for M=%d\n", Split_K, M);
         return tcsl_error_invalid_value();
     }
+    const int ldb = o.ldb ? static_cast<int>(o.ldb) : K;
+    const long ldc = o.ldc ? o.ldc : M;
     // optional events bracket the main kernel only (not the reduction)
     int rc = 0;
-    if (ev_begin && (rc = tcsl_event_record(ev_begin, stream)) != 0)
+    if (o.ev_begin && (rc = tcsl_event_record(o.ev_begin, stream)) != 0)
         return rc;
-    rc = launch_main(stream, Compressed_A, TileOffsets, B, Split_K == 1 ? C : Reduction_Workspace, M, N, K, Split_K,
-                     row_major, forced);
+    if (Split_K == 1)  // the kernel writes C itself, with C's stride and the clamp
+        rc = launch_main(stream, Compressed_A, TileOffsets, B, C, M, N, K, 1, o, ldb, static_cast<int>(ldc), o.relu);
+    else               // dense slabs of partial sums; stride and clamp are applied by the reduction
+        rc = launch_main(stream, Compressed_A, TileOffsets, B, Reduction_Workspace, M, N, K, Split_K, o, ldb, M, false);
     if (rc != 0)
         return rc;
-    if (ev_end && (rc = tcsl_event_record(ev_end, stream)) != 0)
+    if (o.ev_end && (rc = tcsl_event_record(o.ev_end, stream)) != 0)
         return rc;
     if (Split_K == 1)
         return 0;
-    return tcsl_launch_reduce(stream, C, Reduction_Workspace, static_cast<long>(M) * N, Split_K);
+    if (o.row_major || ldc == M)  // C is as dense as the slabs: one flat vector
+        return tcsl_launch_reduce(stream, C, Reduction_Workspace, static_cast<long>(M) * N, 1, static_cast<long>(M) * N,
+                                  Split_K, o.relu ? 1 : 0);
+    return tcsl_launch_reduce(stream, C, Reduction_Workspace, M, N, ldc, Split_K, o.relu ? 1 : 0);
 }
 }  // namespace
 

@@ -158,6 +158,8 @@ __device__ __forceinline__ void clear_tile(uint8_t* tile, int lane)
         *reinterpret_cast<u64_a*>(tile + u * (kWave * 8) + lane * 8) = 0;
 }
 
+// ldb = elements between two tokens' vectors in B, ldo = the same for the output (column-major
+// only; the slabs of partial sums use M); relu != 0 clamps the output at zero (final results only).
 // blockDim.x = W * 64.  Wave w of workgroup g owns tile row (g % groups) * W + w of batch
 // g / groups, groups = ceil(tile rows / W).  NB = number of 16-token column blocks;
 // ROWMAJ = B is [K][N] and the output [M][N].  HALF = N is 8 (the upper eight columns of the single block are computed on duplicates
@@ -170,7 +172,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
                                                                 const int* __restrict__ offsets,
                                                                 const _Float16* __restrict__ B,
                                                                 _Float16* __restrict__ out, int M, int N, int K,
-                                                                int split_k)
+                                                                int split_k, int ldb, int ldo, int relu)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int VPL = kVecPerLane;
@@ -224,7 +226,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
         const int ngran = ntile * NTOK * 8;
         for (int id = threadIdx.x; id < ngran; id += blockDim.x) {
             const int j = id / (NTOK * 8), t = (id >> 3) % NTOK, g = id & 7;
-            const half8 v = *reinterpret_cast<const half8*>(B + (size_t)t * K + (size_t)(kb0 + j) * kTileCols + g * 8);
+            const half8 v = *reinterpret_cast<const half8*>(B + (size_t)t * ldb + (size_t)(kb0 + j) * kTileCols + g * 8);
             *reinterpret_cast<half8*>(bslice + (size_t)j * (NTOK * 128) + t * 128 + ((g ^ (t & 7)) << 4)) = v;
         }
     }
@@ -274,7 +276,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
         int tok = c * 16 + l15;
         if (HALF)
             tok &= 7;
-        bptr[c] = ROWMAJ ? B : B + (size_t)tok * K + (size_t)kb0 * kTileCols + q * 8;
+        bptr[c] = ROWMAJ ? B : B + (size_t)tok * ldb + (size_t)kb0 * kTileCols + q * 8;
 #pragma unroll
         for (int s = 0; s < 2; s++)
             b_off[c][s] = tok * 128 + (((s * 4 + q) ^ (tok & 7)) << 4);
@@ -512,7 +514,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
                 half4 h;
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    h[i] = static_cast<_Float16>(sum[i]);
+                    h[i] = static_cast<_Float16>(relu ? fmaxf(sum[i], 0.f) : sum[i]);
                 // rows r*16 + 4*q .. +3 of token c*16 + l15
                 if (!(HALF && l15 >= 8)) {
                     if (ROWMAJ) {
@@ -520,7 +522,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
                         for (int i = 0; i < 4; i++)  // the 16 tokens of a row are adjacent
                             oslab[(r * 16 + q * 4 + i) * NTOK + c * 16 + l15] = h[i];
                     } else {  // the four q-lanes of a token cover 32 bytes
-                        *reinterpret_cast<half4*>(oslab + (size_t)(c * 16 + l15) * M + r * 16 + q * 4) = h;
+                        *reinterpret_cast<half4*>(oslab + (size_t)(c * 16 + l15) * ldo + r * 16 + q * 4) = h;
                     }
                 }
             }
@@ -538,7 +540,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
 #pragma unroll
                     for (int i = 0; i < 4; i++)
                         *reinterpret_cast<_Float16*>(tile + ((r * 16 + q * 4 + i) * NTOK + c * 16 + l15) * 2) =
-                            static_cast<_Float16>(acc[c][r][i]);
+                            static_cast<_Float16>(relu ? fmaxf(acc[c][r][i], 0.f) : acc[c][r][i]);
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // other lanes read what this lane wrote
 #pragma unroll
@@ -561,7 +563,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
                 half4 h;
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    h[i] = static_cast<_Float16>(acc[c][r][i]);
+                    h[i] = static_cast<_Float16>(relu ? fmaxf(acc[c][r][i], 0.f) : acc[c][r][i]);
                 *reinterpret_cast<half4*>(tile + l15 * kTokStride + (r * 16 + q * 4) * 2) = h;
             }
         }
@@ -573,16 +575,17 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
             const int e = i * kWave + lane;
             const int tok = e >> 4, part = e & 15;
             const half8 v = *reinterpret_cast<const half8*>(tile + tok * kTokStride + part * 16);
-            *reinterpret_cast<half8*>(oslab + (size_t)(c * 16 + tok) * M + part * 8) = v;
+            *reinterpret_cast<half8*>(oslab + (size_t)(c * 16 + tok) * ldo + part * 8) = v;
         }
     }
 }
 
-// C[e] = fp16(sum over slabs of float(W[s][e])) (csrc/Reduction_Kernel.cuh:36-46), 8 elements
-// per thread.  The slab loads of a thread are independent; they are issued eight at a time
-// so their latencies overlap (the reduction is latency bound: a few MB in all).
+// C[n][m] = fp16(sum over slabs of float(W[s][n][m])) (csrc/Reduction_Kernel.cuh:36-46), 8 elements
+// per thread; rows8 = vector length / 8, ldc = elements between two vectors of C (slabs are
+// dense).  The slab loads of a thread are independent; they are issued eight at a time so
+// their latencies overlap (the reduction is latency bound: a few MB in all).
 __global__ __launch_bounds__(64) void tcsl_reduce_kernel(_Float16* __restrict__ C, const _Float16* __restrict__ W,
-                                                        long mn8, long mn, int split_k)
+                                                        long mn8, long mn, int rows8, long ldc, int split_k, int relu)
 {
     const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= mn8)
@@ -610,8 +613,9 @@ __global__ __launch_bounds__(64) void tcsl_reduce_kernel(_Float16* __restrict__ 
     half8 o;
 #pragma unroll
     for (int j = 0; j < 8; j++)
-        o[j] = static_cast<_Float16>(sum[j]);
-    *reinterpret_cast<half8*>(C + i * 8) = o;
+        o[j] = static_cast<_Float16>(relu ? fmaxf(sum[j], 0.f) : sum[j]);
+    const long n = i / rows8, m8 = i - n * rows8;
+    *reinterpret_cast<half8*>(C + n * ldc + m8 * 8) = o;
 }
 
 // Plain streaming copy, used only to calibrate hardware counters against a
@@ -624,7 +628,7 @@ __global__ __launch_bounds__(256) void tcsl_copy_kernel(u32x4* __restrict__ dst,
 
 template<int NB, bool HALF, bool BLDS, bool KSPLIT, bool ROWMAJ, int MAXW>
 int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const void* B, void* out, int M, int N,
-                int K, int split_k, int waves, unsigned lds_bytes)
+                int K, int split_k, int waves, unsigned lds_bytes, int ldb, int ldo, int relu)
 {
     if (waves < 1 || waves > MAXW || lds_bytes > kMaxLdsBytes)
         return static_cast<int>(hipErrorInvalidValue);
@@ -646,7 +650,7 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
     const int groups = KSPLIT ? row_tiles : (row_tiles + waves - 1) / waves;
     hipLaunchKernelGGL(kernel, dim3(groups * split_k), dim3(waves * kWave), lds_bytes, stream,
                        static_cast<const u32x4*>(items), offsets, static_cast<const _Float16*>(B),
-                       static_cast<_Float16*>(out), M, N, K, split_k);
+                       static_cast<_Float16*>(out), M, N, K, split_k, ldb, ldo, relu);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -662,9 +666,10 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
 //         add their results up in LDS (stage_b must be 0).
 // row_major: B is [K][N] and the output [M][N] instead of [N][K] and [N][M] (stage_b must be 0).
 // waves = 1..8 for N <= 32, 1..4 for N = 64; lds_bytes = what the shape needs (the host plans it).
+// ldb, ldo: token strides of B and of the output in elements (column-major; multiples of 8).
 extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offsets, const void* B, void* out, int M,
                                 int N, int K, int split_k, int mode, int waves, int stage_b, int row_major,
-                                unsigned lds_bytes)
+                                unsigned lds_bytes, int ldb, int ldo, int relu)
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (mode != 0 && mode != 1)
@@ -672,7 +677,7 @@ extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offs
     if (stage_b && (mode == 1 || row_major || N > 16))
         return static_cast<int>(hipErrorInvalidValue);
 #define TCSL_GO(NB, HALF, BLDS, KS, RM, MAXW) \
-    launch_spmm<NB, HALF, BLDS, KS, RM, MAXW>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes)
+    launch_spmm<NB, HALF, BLDS, KS, RM, MAXW>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes, ldb, ldo, relu)
 #define TCSL_PICK(NB, HALF, MAXW)                                                                     \
     (row_major ? (mode ? TCSL_GO(NB, HALF, false, true, true, MAXW) : TCSL_GO(NB, HALF, false, false, true, MAXW)) \
                : (mode ? TCSL_GO(NB, HALF, false, true, false, MAXW) : TCSL_GO(NB, HALF, false, false, false, MAXW)))
@@ -692,14 +697,18 @@ extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offs
 #undef TCSL_GO
 }
 
-extern "C" int tcsl_launch_reduce(void* stream, void* C, const void* W, long mn, int split_k)
+// C[n*ldc + m] = sum over slabs of W[s][n*rows + m], n < vectors, m < rows (rows % 8 == 0, ldc % 8 == 0)
+extern "C" int tcsl_launch_reduce(void* stream, void* C, const void* W, long rows, long vectors, long ldc, int split_k,
+                                  int relu)
 {
+    const long mn = rows * vectors;
     const long mn8 = mn / 8;
     const long blocks = (mn8 + 63) / 64;
-    if (blocks < 1 || blocks > 0x7fffffffL)
+    if (blocks < 1 || blocks > 0x7fffffffL || rows / 8 > 0x7fffffffL)
         return static_cast<int>(hipErrorInvalidValue);
     hipLaunchKernelGGL(tcsl_reduce_kernel, dim3((unsigned)blocks), dim3(64), 0, static_cast<hipStream_t>(stream),
-                       static_cast<_Float16*>(C), static_cast<const _Float16*>(W), mn8, mn, split_k);
+                       static_cast<_Float16*>(C), static_cast<const _Float16*>(W), mn8, mn, static_cast<int>(rows / 8),
+                       ldc, split_k, relu);
     return static_cast<int>(hipGetLastError());
 }
 

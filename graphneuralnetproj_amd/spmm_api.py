@@ -34,6 +34,7 @@ EXPORTED_SYMBOLS = (
     "SpMM_PlanLaunch",
     "SpMM_SplitK_API_Planned",
     "SpMM_SplitK_API_RowMajor",
+    "SpMM_SplitK_API_Strided",
     "SpMM_SynthWeights",
     "SpMM_SynthActivations",
     "SpMM_CalibrationCopy",
@@ -106,6 +107,9 @@ def load_library():
     lib.SpMM_SplitK_API_Planned.restype = ctypes.c_int
     lib.SpMM_SplitK_API_Planned.argtypes = ([ctypes.c_void_p] * 5 + [ctypes.c_int] * 3 + [ctypes.c_void_p]
                                             + [ctypes.c_int] * 5)
+    lib.SpMM_SplitK_API_Strided.restype = ctypes.c_int
+    lib.SpMM_SplitK_API_Strided.argtypes = ([ctypes.c_void_p] * 4 + [ctypes.c_long, ctypes.c_void_p, ctypes.c_long]
+                                            + [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_int, ctypes.c_int])
     lib.SpMM_SplitK_API_RowMajor.restype = ctypes.c_int
     lib.SpMM_SplitK_API_RowMajor.argtypes = lib.SpMM_SplitK_API.argtypes
     lib.SpMM_SynthWeights.restype = None
@@ -205,6 +209,23 @@ def SpMM_SplitK_API_RowMajor(stream, A, Compressed_A, TileOffsets, B, C, M_Globa
                                       _ptr(Reduction_Workspace), Split_K)
     if rc != 0:
         raise SpMMError("SpMM_SplitK_API_RowMajor", rc, lib.SpMM_GetErrorString(rc).decode())
+    return rc
+
+
+SPMM_FLAG_RELU = 1
+
+
+def SpMM_SplitK_API_Strided(stream, Compressed_A, TileOffsets, B, ldb, C, ldc, M_Global, N_Global, K_Global,
+                            Reduction_Workspace, Split_K, Flags=0):
+    """Column-major SpMM on token vectors ldb / ldc elements apart, optionally clamped at zero."""
+    lib = load_library()
+    if stream is not None and not isinstance(stream, int):
+        stream = stream.cuda_stream
+    rc = lib.SpMM_SplitK_API_Strided(ctypes.c_void_p(stream) if stream else None, _ptr(Compressed_A), _ptr(TileOffsets),
+                                     _ptr(B), ldb, _ptr(C), ldc, M_Global, N_Global, K_Global,
+                                     _ptr(Reduction_Workspace), Split_K, Flags)
+    if rc != 0:
+        raise SpMMError("SpMM_SplitK_API_Strided", rc, lib.SpMM_GetErrorString(rc).decode())
     return rc
 
 

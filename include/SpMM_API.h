@@ -88,6 +88,20 @@ SPMM_EXPORT int SpMM_SplitK_API_RowMajor(void* stream, const void* A, const void
                                          void* Reduction_Workspace, int Split_K);
 
 /*
+ * SpMM_SplitK_API (column-major operands) for activations and results that sit inside
+ * wider per-token buffers, with an optional fused clamp: B[n*ldb + k], C[n*ldc + m],
+ * ldb >= K, ldc >= M, both multiples of 8 elements; Flags = 0 or SPMM_FLAG_RELU
+ * (C = max(A*B, 0)).  This is what chaining the layers of a decoder block needs without
+ * copies: the attention output projection reads a slice of the fused QKV result, and the
+ * first feed-forward product is followed by ReLU (third_party/ft.patch:513-632 runs that
+ * activation as a separate kernel).  hipErrorInvalidValue for strides that do not fit.
+ */
+#define SPMM_FLAG_RELU 1
+SPMM_EXPORT int SpMM_SplitK_API_Strided(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
+                                        long ldb, void* C, long ldc, int M_Global, int N_Global, int K_Global,
+                                        void* Reduction_Workspace, int Split_K, int Flags);
+
+/*
  * SpMM_SplitK_API with two hipEvent_t recorded on `stream` immediately before and
  * after the main kernel (the split-K reduction, if any, follows KernelEnd), so a
  * benchmark can time that kernel alone inside its own loop.  Either event may be

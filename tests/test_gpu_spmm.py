@@ -378,3 +378,41 @@ def test_row_major_layout_probe(spmm, oracle):
     C = d_C.cpu().numpy()
     for n, k in enumerate(ks):
         assert np.array_equal(C[:, n], A[:, k])
+
+
+@pytest.mark.parametrize("N,split_k,relu", [(16, 1, 0), (16, 4, 1), (8, 1, 1), (32, 2, 0), (64, 1, 1), (16, 3, 0)])
+def test_strided_operands_and_fused_relu(spmm, oracle, N, split_k, relu):
+    """B and C live inside wider per-token buffers; everything outside C's window must stay untouched."""
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    M, K = 512, 1024
+    ldb, ldc, boff, coff = 3 * K, M + 256, K, 128  # B = the middle third of a fused buffer
+    A, B, items, offsets = make_case(spmm, M, K, N, 0.8, seed=11 * N + split_k)
+    ref = oracle.gemm_f32(A, B)
+    if relu:
+        ref = np.maximum(ref, 0.0)
+    wide_B = spmm.synth_activations(N, ldb, seed=5)  # junk around the real activations
+    wide_B[:, boff:boff + K] = B
+    d_items = torch.from_numpy(items.view(np.int32).copy()).to(dev)
+    d_offs = torch.from_numpy(offsets.copy()).to(dev)
+    d_B = torch.from_numpy(wide_B.view(np.int16).copy()).to(dev)
+    d_C = torch.full((N, ldc), -7.0, dtype=torch.float16, device=dev)
+    d_W = torch.full((split_k, N, M), float("nan"), dtype=torch.float16, device=dev) if split_k > 1 else None
+    print(f"[gpu case] strided M={M} N={N} K={K} split_k={split_k} relu={relu}", flush=True)
+    spmm.SpMM_SplitK_API_Strided(torch.cuda.current_stream(), d_items, d_offs, d_B.data_ptr() + 2 * boff, ldb,
+                                 d_C.data_ptr() + 2 * coff, ldc, M, N, K, d_W, split_k,
+                                 spmm.SPMM_FLAG_RELU if relu else 0)
+    torch.cuda.synchronize()
+    C = d_C.cpu().numpy()
+    assert_close(C[:, coff:coff + M], ref)
+    assert (C[:, :coff] == -7.0).all() and (C[:, coff + M:] == -7.0).all()
+    if relu:
+        assert (C[:, coff:coff + M] >= 0).all()
+
+
+def test_strided_rejects_bad_strides(spmm):
+    torch = _torch()
+    z = torch.zeros(1024, dtype=torch.int32, device="cuda:0")
+    for (ldb, ldc, flags) in [(1000, 1024, 0), (1024, 1000, 0), (1028, 1024, 0), (1024, 1028, 0), (1024, 1024, 2)]:
+        with pytest.raises(spmm.SpMMError):
+            spmm.SpMM_SplitK_API_Strided(None, z, z, z, ldb, z, ldc, 1024, 16, 1024, z, 1, flags)
