@@ -1,0 +1,181 @@
+#!/usr/bin/env python3
+"""A stack of decoder-block linear layers on Tiled-CSL weights, chained without copies.
+
+Per layer, with hidden size h and N tokens (all buffers one contiguous vector per token):
+
+    qkv = W_qkv x            (3h x h)      x:   [N][h]
+    o   = W_out qkv[:, :h]   (h x h)       the projection reads the first third of the fused buffer
+    f   = relu(W_ffn1 o)     (4h x h)      clamp fused into the product
+    x'  = W_ffn2 f           (h x 4h)      input of the next layer
+
+This is the sequence of sparse products FasterTransformer's patched OPT decoder issues per token
+(third_party/ft.patch:513-632 feed-forward, :1248-1339 attention projections) with everything
+between them (attention itself, biases, layer norms) left out: a linear-stack microbenchmark
+of the weight stream, sized so that the weights of all layers stay resident in HBM.
+
+    python -m graphneuralnetproj_amd.decoder_stack --hidden 9216 --layers 64 --tokens 16
+
+prints one JSON line with the time per token step for the whole stack, eager and as a HIP graph.
+"""
+import argparse
+import json
+import time
+
+import numpy as np
+
+
+class Layer:
+    """Device-resident encoded weights of one block: name -> (items, offsets, M, K, split_k)."""
+
+    def __init__(self, mats):
+        self.mats = mats
+
+    def clone(self):
+        return Layer({k: (it.clone(), of, M, K, s) for k, (it, of, M, K, s) in self.mats.items()})
+
+    def bytes(self):
+        return sum(it.numel() * 4 for it, _, _, _, _ in self.mats.values())
+
+
+def layer_shapes(h):
+    return {"qkv": (3 * h, h), "out": (h, h), "ffn1": (4 * h, h), "ffn2": (h, 4 * h)}
+
+
+def build_layer(G, torch, dev, h, N, sparsity, seed, keep_dense=False, weight_scale=1.0):
+    """Synthesise, encode and upload one block; weight_scale multiplies the N(0, 0.02) weights."""
+    mats, dense = {}, {}
+    for i, (name, (M, K)) in enumerate(layer_shapes(h).items()):
+        A = G.synth_weights(M, K, sparsity, False, seed=seed * 16 + i)
+        if weight_scale != 1.0:
+            A = (A.astype(np.float32) * weight_scale).astype(np.float16)
+        items, offsets = G.InitSparseMatrixA_API(A)
+        mats[name] = (torch.from_numpy(items.view(np.int32)).to(dev), torch.from_numpy(offsets).to(dev), M, K,
+                      G.SpMM_SuggestSplitK(M, N, K))
+        if keep_dense:
+            dense[name] = A
+    return Layer(mats), dense
+
+
+class Stack:
+    def __init__(self, G, torch, layers, h, N):
+        self.G, self.torch, self.layers, self.h, self.N = G, torch, layers, h, N
+        dev = layers[0].mats["qkv"][0].device
+        f16 = torch.float16
+        self.x = [torch.zeros((N, h), dtype=f16, device=dev) for _ in range(2)]  # ping-pong layer inputs
+        self.qkv = torch.zeros((N, 3 * h), dtype=f16, device=dev)
+        self.o = torch.zeros((N, h), dtype=f16, device=dev)
+        self.f = torch.zeros((N, 4 * h), dtype=f16, device=dev)
+        max_split = max(s for L in layers for (_, _, _, _, s) in L.mats.values())
+        # one workspace for every product, as the reference's caller keeps (third_party/ft.patch:2762-2765)
+        self.ws = torch.zeros((max_split, N, 4 * h), dtype=f16, device=dev)
+
+    def step(self, stream):
+        """Enqueue one token step through every layer; returns the buffer holding the result."""
+        G, h, N = self.G, self.h, self.N
+        cur = 0
+        for L in self.layers:
+            m = L.mats
+            x, nxt = self.x[cur], self.x[cur ^ 1]
+            it, of, M, K, s = m["qkv"]
+            G.SpMM_SplitK_API_Strided(stream, it, of, x, h, self.qkv, 3 * h, M, N, K, self.ws, s, 0)
+            it, of, M, K, s = m["out"]
+            G.SpMM_SplitK_API_Strided(stream, it, of, self.qkv, 3 * h, self.o, h, M, N, K, self.ws, s, 0)
+            it, of, M, K, s = m["ffn1"]
+            G.SpMM_SplitK_API_Strided(stream, it, of, self.o, h, self.f, 4 * h, M, N, K, self.ws, s, G.SPMM_FLAG_RELU)
+            it, of, M, K, s = m["ffn2"]
+            G.SpMM_SplitK_API_Strided(stream, it, of, self.f, 4 * h, nxt, h, M, N, K, self.ws, s, 0)
+            cur ^= 1
+        return self.x[cur]
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--hidden", type=int, default=9216, help="h; 9216 = OPT-66B, 7168 = OPT-30B")
+    ap.add_argument("--layers", type=int, default=64)
+    ap.add_argument("--tokens", type=int, default=16)
+    ap.add_argument("--sparsity", type=float, default=0.8)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--distinct-weights", action="store_true",
+                    help="synthesise and encode every layer separately (default: one layer, copied in HBM)")
+    args = ap.parse_args()
+
+    import torch
+
+    import graphneuralnetproj_amd as G
+
+    G.load_library()
+    dev = torch.device("cuda:0")
+    h, N = args.hidden, args.tokens
+    t0 = time.perf_counter()
+    first, _ = build_layer(G, torch, dev, h, N, args.sparsity, seed=1)
+    layers = [first]
+    for i in range(1, args.layers):
+        layers.append(build_layer(G, torch, dev, h, N, args.sparsity, seed=1 + i)[0] if args.distinct_weights
+                      else first.clone())
+    torch.cuda.synchronize()
+    prep_s = time.perf_counter() - t0
+    stack = Stack(G, torch, layers, h, N)
+    x0 = torch.from_numpy(G.synth_activations(N, h, seed=99).view(np.int16)).to(dev).view(torch.float16)
+    stream = torch.cuda.current_stream()
+
+    def run_eager():
+        stack.x[0].copy_(x0)
+        return stack.step(stream)
+
+    for _ in range(args.warmup):
+        run_eager()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        stack.step(stream)  # chained on the previous step's output: same work, no reset copy
+    torch.cuda.synchronize()
+    eager_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    graph_ms = None
+    graph_matches = None
+    try:
+        want = run_eager().clone()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        stack.x[0].copy_(x0)
+        with torch.cuda.graph(g):
+            out = stack.step(torch.cuda.current_stream())
+        for _ in range(3):  # replays checked against the eager result, with eager work in between
+            stack.x[0].copy_(x0)
+            g.replay()
+            torch.cuda.synchronize()
+            graph_matches = bool(torch.equal(out, want))
+            if not graph_matches:
+                break
+            run_eager()
+            torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            g.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    except Exception as e:  # graph capture is an optimisation; the eager figure stands on its own
+        graph_matches = f"capture failed: {e}"
+
+    weight_bytes = sum(L.bytes() for L in layers)
+    best_ms = min(eager_ms, graph_ms) if graph_ms and graph_matches is True else eager_ms
+    flops = 2.0 * N * sum(M * K for (M, K) in layer_shapes(h).values()) * args.layers
+    print(json.dumps({
+        "metric": "decoder linear stack: time per token step",
+        "value": best_ms, "unit": "ms", "higher_is_better": False,
+        "eager_ms": eager_ms, "graph_ms": graph_ms, "graph_matches_eager": graph_matches,
+        "config": {"workload": f"{args.layers} layers x (QKV, out-proj, FFN1+ReLU, FFN2), h={h}, N={N}, "
+                               f"{args.sparsity * 100:.0f}% sparse",
+                   "weights": "distinct per layer" if args.distinct_weights else "one layer's weights copied per layer"},
+        "resident_weight_bytes": weight_bytes,
+        "hbm_gbps": weight_bytes / (best_ms * 1e-3) / 1e9,
+        "hbm_frac_of_peak": weight_bytes / (best_ms * 1e-3) / 1e9 / 8000.0,
+        "effective_tflops": flops / (best_ms * 1e-3) / 1e12,
+        "hbm_floor_ms": weight_bytes / 8e12 * 1e3,
+        "prep_s": prep_s, "data": "synthetic",
+    }))
+
+
+if __name__ == "__main__":
+    main()

@@ -416,3 +416,36 @@ def test_strided_rejects_bad_strides(spmm):
     for (ldb, ldc, flags) in [(1000, 1024, 0), (1024, 1000, 0), (1028, 1024, 0), (1024, 1028, 0), (1024, 1024, 2)]:
         with pytest.raises(spmm.SpMMError):
             spmm.SpMM_SplitK_API_Strided(None, z, z, z, ldb, z, ldc, 1024, 16, 1024, z, 1, flags)
+
+
+def test_decoder_stack_matches_cpu_chain(spmm, oracle):
+    """Three chained blocks (QKV -> out-proj on a slice -> FFN1+ReLU -> FFN2) against the same chain on the CPU."""
+    torch = _torch()
+    from graphneuralnetproj_amd import decoder_stack as DS
+
+    dev = torch.device("cuda:0")
+    h, N, nlayers = 512, 16, 3
+    layers, dense = [], []
+    for i in range(nlayers):
+        L, d = DS.build_layer(spmm, torch, dev, h, N, 0.6, seed=40 + i, keep_dense=True, weight_scale=4.0)
+        layers.append(L)
+        dense.append(d)
+    stack = DS.Stack(spmm, torch, layers, h, N)
+    x0 = spmm.synth_activations(N, h, seed=99)
+    stack.x[0].copy_(torch.from_numpy(x0.view(np.int16)).to(dev).view(torch.float16))
+    print(f"[gpu case] decoder stack h={h} N={N} layers={nlayers}", flush=True)
+    out = stack.step(torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+
+    x = x0
+    f16 = lambda a: a.astype(np.float16)
+    for d in dense:
+        qkv = f16(oracle.gemm_f32(d["qkv"], x))
+        o = f16(oracle.gemm_f32(d["out"], np.ascontiguousarray(qkv[:, :h])))
+        f = f16(np.maximum(oracle.gemm_f32(d["ffn1"], o), 0.0))
+        x = f16(oracle.gemm_f32(d["ffn2"], f))
+    assert np.abs(x.astype(np.float32)).max() > 1e-3, "the reference chain must not have collapsed to zero"
+    # each product is within the per-call tolerance; four roundings per layer compound, so allow 3x
+    err = np.abs(got.astype(np.float32) - x.astype(np.float32))
+    assert (err <= 3 * (ATOL + RTOL * np.abs(x.astype(np.float32)))).all(), err.max()
