@@ -331,13 +331,8 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
         const uint64_t base = reinterpret_cast<uint64_t>(items + s.begin);
         // descriptor over exactly this segment (nothing at all past the end of the unit)
         i32x4 rs = {(int)(uint32_t)base, (int)((uint32_t)(base >> 32) & 0xffff), live ? s.n * 16 : 0, 0x00020000};
-        static_for<VPL>([&](auto uc) {
-            constexpr int u = decltype(uc)::value;
-            if constexpr (u < 4)
-                regs[slot][u] = load_words<u * 1024>(rs, voff_lo);
-            else
-                regs[slot][u] = load_words<(u - 4) * 1024>(rs, voff_hi);
-        });
+        // Activation loads go first: they hit in L2 and return quickly, and loads return in order,
+        // so behind the weight loads they would hold their slots for a full HBM round trip (1-3 %).
         if (!BLDS) {
             const int bt = live ? s.tile : ntile - 1;
             if (ROWMAJ) {
@@ -354,6 +349,13 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
                         bfrag[slot][cb * 2 + k] = load_activations(bptr[cb] + bt * kTileCols + k * 32);
             }
         }
+        static_for<VPL>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            if constexpr (u < 4)
+                regs[slot][u] = load_words<u * 1024>(rs, voff_lo);
+            else
+                regs[slot][u] = load_words<(u - 4) * 1024>(rs, voff_hi);
+        });
     };
 
     // Waits for every load of `slot` (at most Y younger ones may stay in flight) and keeps the
