@@ -8,6 +8,7 @@ from .spmm_api import (  # noqa: F401
     SpMM_SplitK_API_RowMajor,
     SpMM_SplitK_API_Strided,
     SPMM_FLAG_RELU,
+    SPMM_FLAG_SEPARATE_REDUCTION,
     SpMM_SuggestSplitK,
     SpMMError,
     build_library,

@@ -4,6 +4,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <mutex>
 
 #include "../../include/SpMM_API.h"
 #include "launch_plan.h"
@@ -12,7 +13,7 @@
 extern "C" {
 int tcsl_launch_spmm(void* stream, const void* items, const int* offsets, const void* B, void* out, int M, int N,
                      int K, int split_k, int mode, int waves, int stage_b, int row_major, unsigned lds_bytes, int ldb,
-                     int ldo, int relu);
+                     int ldo, int relu, void* fused_out, int ldc, int fuse_page);
 int tcsl_launch_reduce(void* stream, void* C, const void* W, long rows, long vectors, long ldc, int split_k, int relu);
 int tcsl_launch_copy(void* stream, void* dst, const void* src, long bytes);
 void* tcsl_event_create(void);
@@ -70,23 +71,58 @@ tcsl::LaunchPlan cached_plan(int M, int N, int K, int Split_K, bool row_major)
     return p;
 }
 
+// The fused split-K reduction counts arrivals in one of 64 pages of device counters.  Calls on
+// one stream run in order and can share a page; calls on different streams may overlap, so each
+// stream gets a page of its own, first come first served.  -1 when all pages are taken (the call
+// then uses the separate reduction kernel).
+int counter_page(void* stream)
+{
+    constexpr int kPages = 64;
+    static std::mutex mu;
+    static void* owner[kPages];
+    static int used = 0;
+    std::lock_guard<std::mutex> lock(mu);
+    for (int i = 0; i < used; i++)
+        if (owner[i] == stream)
+            return i;
+    if (used == kPages)
+        return -1;
+    owner[used] = stream;
+    return used++;
+}
+
 // What varies between the entry points that end in the same two launches.
 struct CallOptions {
     bool row_major = false;   // B is [K][N], C and the slabs [M][N]
     long ldb = 0;             // elements between two tokens' vectors in B (0 = K); column-major only
     long ldc = 0;             // the same for C (0 = M)
     bool relu = false;        // clamp C at zero
+    bool separate_reduction = false;  // never fuse the reduction into the main kernel
     void* ev_begin = nullptr; // events recorded around the main kernel
     void* ev_end = nullptr;
     const tcsl::LaunchPlan* forced = nullptr;
 };
 
+// fused_out != nullptr asks for the fused reduction; *fused says whether it was possible.
 int launch_main(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* out, int M, int N,
-                int K, int Split_K, const CallOptions& o, int ldb, int ldo, bool relu)
+                int K, int Split_K, const CallOptions& o, int ldb, int ldo, bool relu, void* fused_out, long ldc,
+                bool* fused)
 {
     const tcsl::LaunchPlan p = o.forced ? *o.forced : cached_plan(M, N, K, Split_K, o.row_major);
+    int page = -1;
+    if (fused_out) {
+        const long row_tiles = M / tcsl::kTileRows;
+        const long groups = p.mode ? row_tiles : (row_tiles + p.waves - 1) / p.waves;
+        if (groups <= 4096)
+            page = counter_page(stream);
+    }
+    if (fused)
+        *fused = page >= 0;
     return tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, out, M, N, K, Split_K, p.mode, p.waves, p.stage_b,
-                            o.row_major ? 1 : 0, p.lds_bytes, ldb, ldo, relu ? 1 : 0);
+                            o.row_major ? 1 : 0, p.lds_bytes, ldb, ldo,
+                            relu && (Split_K == 1 || page >= 0) ? 1 : 0,  // slabs of partial sums are never clamped
+                            page >= 0 ? fused_out : nullptr,
+                            static_cast<int>(ldc), page);
 }
 
 int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* C, int M, int N,
@@ -115,12 +151,13 @@ extern "C" int SpMM_SplitK_API_Strided(void* stream, const void* Compressed_A, c
                                        int Split_K, int Flags)
 {
     if (ldb < K || ldc < M || ldb % 8 != 0 || ldc % 8 != 0 || ldb > 0x7fffffffL || ldc > 0x7fffffffL ||
-        (Flags & ~SPMM_FLAG_RELU) != 0)
+        (Flags & ~(SPMM_FLAG_RELU | SPMM_FLAG_SEPARATE_REDUCTION)) != 0)
         return tcsl_error_invalid_value();
     CallOptions o;
     o.ldb = ldb;
     o.ldc = ldc;
     o.relu = (Flags & SPMM_FLAG_RELU) != 0;
+    o.separate_reduction = (Flags & SPMM_FLAG_SEPARATE_REDUCTION) != 0;
     return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, o);
 }
 
@@ -179,7 +216,8 @@ extern "C" int SpMM_SplitK_Partials(void* stream, const void* Compressed_A, cons
         return tcsl_error_invalid_value();
     if (!Compressed_A || !TileOffsets || !B || !Partials)
         return tcsl_error_invalid_value();
-    return launch_main(stream, Compressed_A, TileOffsets, B, Partials, M, N, K, Split_K, CallOptions{}, K, M, false);
+    return launch_main(stream, Compressed_A, TileOffsets, B, Partials, M, N, K, Split_K, CallOptions{}, K, M, false,
+                       nullptr, 0, nullptr);
 }
 
 extern "C" void* SpMM_EventCreate(void)
@@ -231,15 +269,23 @@ int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, 
     int rc = 0;
     if (o.ev_begin && (rc = tcsl_event_record(o.ev_begin, stream)) != 0)
         return rc;
-    if (Split_K == 1)  // the kernel writes C itself, with C's stride and the clamp
-        rc = launch_main(stream, Compressed_A, TileOffsets, B, C, M, N, K, 1, o, ldb, static_cast<int>(ldc), o.relu);
-    else               // dense slabs of partial sums; stride and clamp are applied by the reduction
-        rc = launch_main(stream, Compressed_A, TileOffsets, B, Reduction_Workspace, M, N, K, Split_K, o, ldb, M, false);
+    bool fused = false;
+    if (Split_K == 1) {  // the kernel writes C itself, with C's stride and the clamp
+        rc = launch_main(stream, Compressed_A, TileOffsets, B, C, M, N, K, 1, o, ldb, static_cast<int>(ldc), o.relu,
+                         nullptr, 0, nullptr);
+    } else {
+        // Dense slabs of partial sums; stride and clamp are applied by the reduction, which the
+        // main kernel does itself (its last workgroup per group of rows) unless the caller wants
+        // the main kernel timed alone, the operands are row-major, or no counters are free.
+        const bool want_fused = !o.row_major && !o.separate_reduction && !o.ev_begin && !o.ev_end;
+        rc = launch_main(stream, Compressed_A, TileOffsets, B, Reduction_Workspace, M, N, K, Split_K, o, ldb, M, o.relu,
+                         want_fused ? C : nullptr, ldc, &fused);
+    }
     if (rc != 0)
         return rc;
     if (o.ev_end && (rc = tcsl_event_record(o.ev_end, stream)) != 0)
         return rc;
-    if (Split_K == 1)
+    if (Split_K == 1 || fused)
         return 0;
     if (o.row_major || ldc == M)  // C is as dense as the slabs: one flat vector
         return tcsl_launch_reduce(stream, C, Reduction_Workspace, static_cast<long>(M) * N, 1, static_cast<long>(M) * N,

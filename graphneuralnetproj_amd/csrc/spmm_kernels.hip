@@ -68,6 +68,13 @@ constexpr int kVecPerLane = 8;  // 16-byte vectors per lane and ring slot: 512 v
 constexpr int kRing = 2;        // ring slots: one tile being consumed, one in flight
 constexpr unsigned kMaxLdsBytes = 160 * 1024;  // LDS of one gfx950 compute unit
 
+// Arrival counters of the fused split-K reduction: one page per caller stream, one counter per
+// group of output rows.  Zero when the module is loaded; the workgroup that brings a counter to
+// Split_K sets it back to zero, so every call finds them at zero.
+constexpr int kCounterPages = 64;
+constexpr int kCountersPerPage = 4096;
+__device__ unsigned int tcsl_arrivals[kCounterPages][kCountersPerPage];
+
 template<int... Is, typename F>
 __device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F&& f)
 {
@@ -160,6 +167,9 @@ __device__ __forceinline__ void clear_tile(uint8_t* tile, int lane)
 
 // ldb = elements between two tokens' vectors in B, ldo = the same for the output (column-major
 // only; the slabs of partial sums use M); relu != 0 clamps the output at zero (final results only).
+// fuse_page >= 0 (Split_K > 1, column-major): `out` receives the slabs of partial sums as usual,
+// and the last workgroup to finish a group of rows adds the slabs up into fused_out (token stride
+// ldc, clamped if relu) itself; arrivals are counted in tcsl_arrivals[fuse_page].
 // blockDim.x = W * 64.  Wave w of workgroup g owns tile row (g % groups) * W + w of batch
 // g / groups, groups = ceil(tile rows / W).  NB = number of 16-token column blocks;
 // ROWMAJ = B is [K][N] and the output [M][N].  HALF = N is 8 (the upper eight columns of the single block are computed on duplicates
@@ -172,7 +182,9 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
                                                                 const int* __restrict__ offsets,
                                                                 const _Float16* __restrict__ B,
                                                                 _Float16* __restrict__ out, int M, int N, int K,
-                                                                int split_k, int ldb, int ldo, int relu)
+                                                                int split_k, int ldb, int ldo, int relu,
+                                                                _Float16* __restrict__ fused_out, int ldc,
+                                                                int fuse_page)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int VPL = kVecPerLane;
@@ -209,7 +221,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
         kb0 = kb0 < kb1 ? kb0 : kb1;
         kb1 = kb0 + run < kb1 ? kb0 + run : kb1;
     }
-    const int ntile = kb1 - kb0;  // tiles of this wave
+    const int ntile = active ? kb1 - kb0 : 0;  // tiles of this wave
     uint8_t* const tile = lds + wave * kTileBytes;
     // Activations in LDS, per tile [token][8 granules of 16 B at position g ^ (token & 7)]: the
     // batch's slice, staged once and shared (BLDS), or (ROWMAJ) a one-tile buffer per wave in
@@ -223,7 +235,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
     int wreg = toff[lane <= ntile ? lane : ntile];
 
     if (BLDS) {
-        const int ngran = ntile * NTOK * 8;
+        const int ngran = (kb1 - kb0) * NTOK * 8;  // the whole batch, whatever this wave's own share
         for (int id = threadIdx.x; id < ngran; id += blockDim.x) {
             const int j = id / (NTOK * 8), t = (id >> 3) % NTOK, g = id & 7;
             const half8 v = *reinterpret_cast<const half8*>(B + (size_t)t * ldb + (size_t)(kb0 + j) * kTileCols + g * 8);
@@ -234,8 +246,9 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
         clear_tile(tile, lane);
     if (BLDS)
         __syncthreads();  // the only barrier: every wave of the workgroup reaches it
-    if (!KSPLIT && !active)
-        return;
+    if (!KSPLIT && !active && fuse_page < 0)
+        return;  // (with the fused reduction every wave has to reach the barriers at the end)
+    const bool clamp = relu && fuse_page < 0;  // partial sums are never clamped
 
     auto tile_range = [&](int i, int& begin, int& end) {  // 0 <= i < ntile
         if (i + 1 - wbase >= kWave) {  // slide the window (more than 63 tiles per wave only)
@@ -484,6 +497,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
             land(s, std::integral_constant<int, 0>{});
     }
 
+    auto write_out = [&]() {
     // Epilogue.  acc[c][r][i] is output row r*16 + 4*q + i of this tile row for token
     // c*16 + l15; the output keeps one contiguous M vector per token.  The block goes through
     // the wave's LDS tile as [token][128 rows] (token stride padded to 272 B) so that the
@@ -516,7 +530,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
                 half4 h;
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    h[i] = static_cast<_Float16>(relu ? fmaxf(sum[i], 0.f) : sum[i]);
+                    h[i] = static_cast<_Float16>(clamp ? fmaxf(sum[i], 0.f) : sum[i]);
                 // rows r*16 + 4*q .. +3 of token c*16 + l15
                 if (!(HALF && l15 >= 8)) {
                     if (ROWMAJ) {
@@ -542,7 +556,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
 #pragma unroll
                     for (int i = 0; i < 4; i++)
                         *reinterpret_cast<_Float16*>(tile + ((r * 16 + q * 4 + i) * NTOK + c * 16 + l15) * 2) =
-                            static_cast<_Float16>(relu ? fmaxf(acc[c][r][i], 0.f) : acc[c][r][i]);
+                            static_cast<_Float16>(clamp ? fmaxf(acc[c][r][i], 0.f) : acc[c][r][i]);
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // other lanes read what this lane wrote
 #pragma unroll
@@ -565,7 +579,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
                 half4 h;
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    h[i] = static_cast<_Float16>(relu ? fmaxf(acc[c][r][i], 0.f) : acc[c][r][i]);
+                    h[i] = static_cast<_Float16>(clamp ? fmaxf(acc[c][r][i], 0.f) : acc[c][r][i]);
                 *reinterpret_cast<half4*>(tile + l15 * kTokStride + (r * 16 + q * 4) * 2) = h;
             }
         }
@@ -580,6 +594,60 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
             *reinterpret_cast<half8*>(oslab + (size_t)(c * 16 + tok) * ldo + part * 8) = v;
         }
     }
+    };
+    if (KSPLIT || active)
+        write_out();
+    if (ROWMAJ || fuse_page < 0)
+        return;
+
+    // Fused split-K reduction.  Every workgroup has just written its slab; the last of the Split_K
+    // workgroups that share a group of rows adds the slabs up, in slab order like the separate
+    // kernel (csrc/Reduction_Kernel.cuh:36-46), so both paths give the same bits.
+    __threadfence();  // this workgroup's partial sums are visible device-wide before it is counted
+    __syncthreads();
+    unsigned int* const counter = &tcsl_arrivals[fuse_page][blockIdx.x % groups];
+    unsigned int* const flag = reinterpret_cast<unsigned int*>(lds);
+    if (threadIdx.x == 0)
+        *flag = atomicAdd(counter, 1u);
+    __syncthreads();
+    if (*flag != static_cast<unsigned int>(split_k - 1))
+        return;
+    __threadfence();  // the other workgroups' partial sums are visible here
+    const int row0 = (KSPLIT ? blockIdx.x % groups : (blockIdx.x % groups) * W) * kTileRows;
+    int nrows = (KSPLIT ? 1 : W) * kTileRows;
+    nrows = nrows < M - row0 ? nrows : M - row0;
+    const int per_tok = nrows / 8;
+    const size_t slab = (size_t)M * N;
+    for (int c = threadIdx.x; c < per_tok * N; c += blockDim.x) {
+        const int tok = c / per_tok, m8 = c - tok * per_tok;
+        const _Float16* w0 = out + (size_t)tok * M + row0 + m8 * 8;
+        float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        int sidx = 0;
+        for (; sidx + 4 <= split_k; sidx += 4) {
+            half8 w[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                w[u] = *reinterpret_cast<const half8*>(w0 + (size_t)(sidx + u) * slab);
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    sum[j] += static_cast<float>(w[u][j]);
+        }
+        for (; sidx < split_k; sidx++) {
+            const half8 w = *reinterpret_cast<const half8*>(w0 + (size_t)sidx * slab);
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                sum[j] += static_cast<float>(w[j]);
+        }
+        half8 o;
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            o[j] = static_cast<_Float16>(relu ? fmaxf(sum[j], 0.f) : sum[j]);
+        *reinterpret_cast<half8*>(fused_out + (size_t)tok * ldc + row0 + m8 * 8) = o;
+    }
+    if (threadIdx.x == 0)
+        *counter = 0;  // ready for the next call
 }
 
 // C[n][m] = fp16(sum over slabs of float(W[s][n][m])) (csrc/Reduction_Kernel.cuh:36-46), 8 elements
@@ -630,7 +698,8 @@ __global__ __launch_bounds__(256) void tcsl_copy_kernel(u32x4* __restrict__ dst,
 
 template<int NB, bool HALF, bool BLDS, bool KSPLIT, bool ROWMAJ, int MAXW>
 int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const void* B, void* out, int M, int N,
-                int K, int split_k, int waves, unsigned lds_bytes, int ldb, int ldo, int relu)
+                int K, int split_k, int waves, unsigned lds_bytes, int ldb, int ldo, int relu, void* fused_out,
+                int ldc, int fuse_page)
 {
     if (waves < 1 || waves > MAXW || lds_bytes > kMaxLdsBytes)
         return static_cast<int>(hipErrorInvalidValue);
@@ -652,7 +721,8 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
     const int groups = KSPLIT ? row_tiles : (row_tiles + waves - 1) / waves;
     hipLaunchKernelGGL(kernel, dim3(groups * split_k), dim3(waves * kWave), lds_bytes, stream,
                        static_cast<const u32x4*>(items), offsets, static_cast<const _Float16*>(B),
-                       static_cast<_Float16*>(out), M, N, K, split_k, ldb, ldo, relu);
+                       static_cast<_Float16*>(out), M, N, K, split_k, ldb, ldo, relu, static_cast<_Float16*>(fused_out), ldc,
+                       fuse_page);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -669,17 +739,26 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
 // row_major: B is [K][N] and the output [M][N] instead of [N][K] and [N][M] (stage_b must be 0).
 // waves = 1..8 for N <= 32, 1..4 for N = 64; lds_bytes = what the shape needs (the host plans it).
 // ldb, ldo: token strides of B and of the output in elements (column-major; multiples of 8).
+// fuse_page >= 0: out = Split_K dense slabs, and the kernel itself reduces them into fused_out
+// (token stride ldc), counting arrivals on that page of counters; at most 4096 row groups.
 extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offsets, const void* B, void* out, int M,
                                 int N, int K, int split_k, int mode, int waves, int stage_b, int row_major,
-                                unsigned lds_bytes, int ldb, int ldo, int relu)
+                                unsigned lds_bytes, int ldb, int ldo, int relu, void* fused_out, int ldc,
+                                int fuse_page)
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (mode != 0 && mode != 1)
         return static_cast<int>(hipErrorInvalidValue);
     if (stage_b && (mode == 1 || row_major || N > 16))
         return static_cast<int>(hipErrorInvalidValue);
+    if (fuse_page >= 0) {
+        const long groups = mode ? M / kTileRows : (M / kTileRows + waves - 1) / waves;
+        if (fuse_page >= kCounterPages || groups > kCountersPerPage || row_major || split_k < 2 || !fused_out)
+            return static_cast<int>(hipErrorInvalidValue);
+    }
 #define TCSL_GO(NB, HALF, BLDS, KS, RM, MAXW) \
-    launch_spmm<NB, HALF, BLDS, KS, RM, MAXW>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes, ldb, ldo, relu)
+    launch_spmm<NB, HALF, BLDS, KS, RM, MAXW>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes, ldb, ldo, relu, \
+                                              fused_out, ldc, fuse_page)
 #define TCSL_PICK(NB, HALF, MAXW)                                                                     \
     (row_major ? (mode ? TCSL_GO(NB, HALF, false, true, true, MAXW) : TCSL_GO(NB, HALF, false, false, true, MAXW)) \
                : (mode ? TCSL_GO(NB, HALF, false, true, false, MAXW) : TCSL_GO(NB, HALF, false, false, false, MAXW)))

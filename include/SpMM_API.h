@@ -61,7 +61,9 @@ SPMM_EXPORT int InitSparseMatrixA_API(const uint16_t* A_h, int M, int N, int K, 
  * only enqueues work on `stream`; it never synchronises.
  *   Split_K == 1: C is written directly, the workspace is not touched.
  *   Split_K  > 1: batch b of ceil((K/64)/Split_K) column tiles writes fp16 partial
- *                 sums to Reduction_Workspace[b*M*N ..), then C = fp16(sum in fp32).
+ *                 sums to Reduction_Workspace[b*M*N ..), then C = fp16(sum in fp32), added
+ *                 up in batch order either by the last workgroup of the same launch to
+ *                 finish a group of rows or by a second kernel (same bits either way).
  *                 Reduction_Workspace must hold Split_K*M*N fp16 values and may be
  *                 shared by successive calls on one stream.
  * Accumulation is fp32.  Returns the hipError_t value: 0 on success;
@@ -69,7 +71,10 @@ SPMM_EXPORT int InitSparseMatrixA_API(const uint16_t* A_h, int M, int N, int K, 
  * {8, 16, 32, 64} (csrc/SpMM_API.cu:192-193); hipErrorInvalidValue for M % 128,
  * K % 64, Split_K < 1 or a null pointer (the reference checks these only in
  * debug builds, :93-98, and requires M % 256).  Nothing is launched on error.
- * Thread safe: no mutable state.
+ * Thread safe.  The in-launch reduction counts arrivals in a small static device array, one
+ * page per stream handle (64 pages; further streams fall back to the second kernel): calls on
+ * one stream never overlap, calls on different streams never share a page.  A call recorded
+ * into a HIP graph keeps the page of the stream it was captured on.
  */
 SPMM_EXPORT int SpMM_SplitK_API(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets, const void* B,
                     void* C, int M_Global, int N_Global, int K_Global, void* Reduction_Workspace, int Split_K);
@@ -90,13 +95,14 @@ SPMM_EXPORT int SpMM_SplitK_API_RowMajor(void* stream, const void* A, const void
 /*
  * SpMM_SplitK_API (column-major operands) for activations and results that sit inside
  * wider per-token buffers, with an optional fused clamp: B[n*ldb + k], C[n*ldc + m],
- * ldb >= K, ldc >= M, both multiples of 8 elements; Flags = 0 or SPMM_FLAG_RELU
- * (C = max(A*B, 0)).  This is what chaining the layers of a decoder block needs without
+ * ldb >= K, ldc >= M, both multiples of 8 elements; Flags = 0 or a sum of SPMM_FLAG_RELU
+ * (C = max(A*B, 0)) and SPMM_FLAG_SEPARATE_REDUCTION.  This is what chaining the layers of a decoder block needs without
  * copies: the attention output projection reads a slice of the fused QKV result, and the
  * first feed-forward product is followed by ReLU (third_party/ft.patch:513-632 runs that
  * activation as a separate kernel).  hipErrorInvalidValue for strides that do not fit.
  */
 #define SPMM_FLAG_RELU 1
+#define SPMM_FLAG_SEPARATE_REDUCTION 2 /* Split_K > 1: always run the reduction as its own kernel */
 SPMM_EXPORT int SpMM_SplitK_API_Strided(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
                                         long ldb, void* C, long ldc, int M_Global, int N_Global, int K_Global,
                                         void* Reduction_Workspace, int Split_K, int Flags);

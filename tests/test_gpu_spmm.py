@@ -413,7 +413,7 @@ def test_strided_operands_and_fused_relu(spmm, oracle, N, split_k, relu):
 def test_strided_rejects_bad_strides(spmm):
     torch = _torch()
     z = torch.zeros(1024, dtype=torch.int32, device="cuda:0")
-    for (ldb, ldc, flags) in [(1000, 1024, 0), (1024, 1000, 0), (1028, 1024, 0), (1024, 1028, 0), (1024, 1024, 2)]:
+    for (ldb, ldc, flags) in [(1000, 1024, 0), (1024, 1000, 0), (1028, 1024, 0), (1024, 1028, 0), (1024, 1024, 4)]:
         with pytest.raises(spmm.SpMMError):
             spmm.SpMM_SplitK_API_Strided(None, z, z, z, ldb, z, ldc, 1024, 16, 1024, z, 1, flags)
 
@@ -449,3 +449,79 @@ def test_decoder_stack_matches_cpu_chain(spmm, oracle):
     # each product is within the per-call tolerance; four roundings per layer compound, so allow 3x
     err = np.abs(got.astype(np.float32) - x.astype(np.float32))
     assert (err <= 3 * (ATOL + RTOL * np.abs(x.astype(np.float32)))).all(), err.max()
+
+
+@pytest.mark.parametrize("M,K,N,split_k", [
+    (1024, 1024, 16, 4), (1024, 1024, 8, 2), (1024, 2048, 32, 8), (1024, 1024, 64, 3),
+    (1152, 1024, 16, 5),      # nine tile rows: a partly filled workgroup in the row-sharing layout
+    (7168, 7168, 16, 4),      # an OPT-30B attention projection, the planner's own choice of split
+])
+def test_fused_reduction_matches_separate_kernel_bit_for_bit(spmm, oracle, M, K, N, split_k):
+    """Split_K > 1: the in-launch reduction and the second-kernel reduction sum the same slabs in the same order."""
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    A, B, items, offsets = make_case(spmm, M, K, N, 0.8, seed=M + 3 * K + N + split_k)
+    d_items = torch.from_numpy(items.view(np.int32).copy()).to(dev)
+    d_offs = torch.from_numpy(offsets.copy()).to(dev)
+    d_B = torch.from_numpy(np.ascontiguousarray(B).view(np.int16).copy()).to(dev)
+    outs = []
+    for flags in (0, spmm.SPMM_FLAG_SEPARATE_REDUCTION, spmm.SPMM_FLAG_RELU,
+                  spmm.SPMM_FLAG_RELU | spmm.SPMM_FLAG_SEPARATE_REDUCTION):
+        d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device=dev)
+        d_W = torch.full((split_k, N, M), float("nan"), dtype=torch.float16, device=dev)
+        print(f"[gpu case] fused-vs-separate M={M} N={N} K={K} split_k={split_k} flags={flags}", flush=True)
+        for _ in range(3):  # repeated calls: the arrival counters must come back to zero every time
+            spmm.SpMM_SplitK_API_Strided(torch.cuda.current_stream(), d_items, d_offs, d_B, K, d_C, M, M, N, K, d_W,
+                                         split_k, flags)
+        torch.cuda.synchronize()
+        outs.append(d_C.cpu().numpy())
+    assert np.array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16))
+    assert np.array_equal(outs[2].view(np.uint16), outs[3].view(np.uint16))
+    if M * K <= 4 * 1024 * 1024:
+        ref = oracle.gemm_f32(A, B)
+        assert_close(outs[0], ref)
+        assert_close(outs[2], np.maximum(ref, 0.0))
+
+
+@pytest.mark.parametrize("mode,waves,stage_b", [(0, 7, 1), (0, 3, 0), (1, 8, 0), (1, 5, 0)])
+def test_fused_reduction_in_every_launch_shape(spmm, oracle, mode, waves, stage_b):
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    M, K, N, split_k = 1152, 1536, 16, 6
+    A, B, items, offsets = make_case(spmm, M, K, N, 0.8, seed=5 + mode + waves)
+    ref = oracle.gemm_f32(A, B)
+    d_items = torch.from_numpy(items.view(np.int32).copy()).to(dev)
+    d_offs = torch.from_numpy(offsets.copy()).to(dev)
+    d_B = torch.from_numpy(np.ascontiguousarray(B).view(np.int16).copy()).to(dev)
+    d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device=dev)
+    d_W = torch.full((split_k, N, M), float("nan"), dtype=torch.float16, device=dev)
+    print(f"[gpu case] fused planned mode={mode} waves={waves} stage={stage_b}", flush=True)
+    for _ in range(2):
+        spmm.SpMM_SplitK_API_Planned(torch.cuda.current_stream(), d_items, d_offs, d_B, d_C, M, N, K, d_W, split_k,
+                                     mode, waves, stage_b, 0)
+    torch.cuda.synchronize()
+    assert_close(d_C.cpu().numpy(), ref)
+
+
+def test_fused_reduction_on_two_streams(spmm, oracle):
+    """Calls that overlap on different streams count their arrivals on different pages."""
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    M, K, N, split_k = 2048, 2048, 16, 4
+    cases = []
+    for i in range(2):
+        A, B, items, offsets = make_case(spmm, M, K, N, 0.8, seed=900 + i)
+        cases.append((oracle.gemm_f32(A, B),
+                      torch.from_numpy(items.view(np.int32).copy()).to(dev), torch.from_numpy(offsets.copy()).to(dev),
+                      torch.from_numpy(np.ascontiguousarray(B).view(np.int16).copy()).to(dev),
+                      torch.full((N, M), float("nan"), dtype=torch.float16, device=dev),
+                      torch.full((split_k, N, M), float("nan"), dtype=torch.float16, device=dev),
+                      torch.cuda.Stream()))
+    torch.cuda.synchronize()
+    print("[gpu case] fused reduction on two streams", flush=True)
+    for _ in range(20):
+        for (_, it, of, b, c, w, st) in cases:
+            spmm.SpMM_SplitK_API(st, None, it, of, b, c, M, N, K, w, split_k)
+    torch.cuda.synchronize()
+    for (ref, _, _, _, c, _, _) in cases:
+        assert_close(c.cpu().numpy(), ref)
