@@ -112,6 +112,38 @@ __device__ __forceinline__ half8 load_activations_at(const _Float16* base, uint3
     return r;
 }
 
+// Stores and loads at system scope (write through every cache level / served from memory):
+// how the slabs of partial sums travel between workgroups of one launch without cache
+// maintenance.  A device-wide fence would write back and invalidate the whole L2 of the XCD,
+// which the weight stream lives in.
+__device__ __forceinline__ void store_through(_Float16* p, half8 v)
+{
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void store_through(_Float16* p, half4 v)
+{
+    asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+}
+// Four independent 16-byte loads from memory; all have arrived when this returns.
+__device__ __forceinline__ void load_through4(const _Float16* p0, const _Float16* p1, const _Float16* p2,
+                                              const _Float16* p3, half8 (&w)[4])
+{
+    asm volatile("global_load_dwordx4 %0, %4, off sc0 sc1\n"
+                 "global_load_dwordx4 %1, %5, off sc0 sc1\n"
+                 "global_load_dwordx4 %2, %6, off sc0 sc1\n"
+                 "global_load_dwordx4 %3, %7, off sc0 sc1\n"
+                 "s_waitcnt vmcnt(0)"
+                 : "=&v"(w[0]), "=&v"(w[1]), "=&v"(w[2]), "=&v"(w[3])
+                 : "v"(p0), "v"(p1), "v"(p2), "v"(p3)
+                 : "memory");
+}
+__device__ __forceinline__ half8 load_through(const _Float16* p)
+{
+    half8 w;
+    asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1\n s_waitcnt vmcnt(0)" : "=&v"(w) : "v"(p) : "memory");
+    return w;
+}
+
 // Wait until at most N vector-memory loads are outstanding (they complete in order).
 template<int N>
 __device__ __forceinline__ void wait_loads()
@@ -538,7 +570,11 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
                         for (int i = 0; i < 4; i++)  // the 16 tokens of a row are adjacent
                             oslab[(r * 16 + q * 4 + i) * NTOK + c * 16 + l15] = h[i];
                     } else {  // the four q-lanes of a token cover 32 bytes
-                        *reinterpret_cast<half4*>(oslab + (size_t)(c * 16 + l15) * ldo + r * 16 + q * 4) = h;
+                        _Float16* dst = oslab + (size_t)(c * 16 + l15) * ldo + r * 16 + q * 4;
+                        if (fuse_page >= 0)
+                            store_through(dst, h);
+                        else
+                            *reinterpret_cast<half4*>(dst) = h;
                     }
                 }
             }
@@ -591,7 +627,11 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
             const int e = i * kWave + lane;
             const int tok = e >> 4, part = e & 15;
             const half8 v = *reinterpret_cast<const half8*>(tile + tok * kTokStride + part * 16);
-            *reinterpret_cast<half8*>(oslab + (size_t)(c * 16 + tok) * ldo + part * 8) = v;
+            _Float16* dst = oslab + (size_t)(c * 16 + tok) * ldo + part * 8;
+            if (fuse_page >= 0)
+                store_through(dst, v);
+            else
+                *reinterpret_cast<half8*>(dst) = v;
         }
     }
     };
@@ -603,16 +643,15 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
     // Fused split-K reduction.  Every workgroup has just written its slab; the last of the Split_K
     // workgroups that share a group of rows adds the slabs up, in slab order like the separate
     // kernel (csrc/Reduction_Kernel.cuh:36-46), so both paths give the same bits.
-    __threadfence();  // this workgroup's partial sums are visible device-wide before it is counted
+    wait_loads<0>();  // this workgroup's partial sums (written through) have reached memory before it is counted
     __syncthreads();
     unsigned int* const counter = &tcsl_arrivals[fuse_page][blockIdx.x % groups];
     unsigned int* const flag = reinterpret_cast<unsigned int*>(lds);
     if (threadIdx.x == 0)
-        *flag = atomicAdd(counter, 1u);
+        *flag = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (*flag != static_cast<unsigned int>(split_k - 1))
         return;
-    __threadfence();  // the other workgroups' partial sums are visible here
     const int row0 = (KSPLIT ? blockIdx.x % groups : (blockIdx.x % groups) * W) * kTileRows;
     int nrows = (KSPLIT ? 1 : W) * kTileRows;
     nrows = nrows < M - row0 ? nrows : M - row0;
@@ -625,9 +664,8 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
         int sidx = 0;
         for (; sidx + 4 <= split_k; sidx += 4) {
             half8 w[4];
-#pragma unroll
-            for (int u = 0; u < 4; u++)
-                w[u] = *reinterpret_cast<const half8*>(w0 + (size_t)(sidx + u) * slab);
+            load_through4(w0 + (size_t)sidx * slab, w0 + (size_t)(sidx + 1) * slab, w0 + (size_t)(sidx + 2) * slab,
+                          w0 + (size_t)(sidx + 3) * slab, w);
 #pragma unroll
             for (int u = 0; u < 4; u++)
 #pragma unroll
@@ -635,7 +673,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
                     sum[j] += static_cast<float>(w[u][j]);
         }
         for (; sidx < split_k; sidx++) {
-            const half8 w = *reinterpret_cast<const half8*>(w0 + (size_t)sidx * slab);
+            const half8 w = load_through(w0 + (size_t)sidx * slab);
 #pragma unroll
             for (int j = 0; j < 8; j++)
                 sum[j] += static_cast<float>(w[j]);
