@@ -4,7 +4,7 @@
 // The reference fixes one block shape and tunes Split_K per matrix by hand
 // (kernel_benchmark/benchmark.sh:15, end2end_inference/ft_tools/huggingface_opt_convert_Phase2.py:20).
 // Here the choice is made by a small analytic model of an MI355X (256 compute units, one
-// workgroup slot set per unit limited by LDS and registers), fitted to a sweep of about 2500
+// workgroup slot set per unit limited by LDS and registers), fitted to a sweep of about 2800
 // measured (shape, N, plan) points on OPT-30B/66B layer shapes at 80 % sparsity, backed by a
 // table of the measured optimum for those shapes themselves.
 #include "launch_plan.h"
@@ -22,20 +22,21 @@ constexpr long kTileLds = 16384;   // dense fp16 image of one 128x64 tile
 constexpr int kCUs = 256;
 
 // Fitted constants (microseconds, bytes per microsecond).
-constexpr double kLaunchUs = 2.87;          // fixed cost of the main kernel
+constexpr double kLaunchUs = 2.04;          // fixed cost of the main kernel
 constexpr double kTileBytes = 6558.0;       // one tile at 80 % sparsity
 constexpr double kChipBytesPerUs = 7.0e6;   // whole-chip stream rate
-constexpr double kCuBytesPerUs = 38.3e3;    // what one compute unit can pull on its own
-constexpr double kWaveTileUs = 0.712;       // a lone wave's turnaround per tile (latency bound)
-constexpr double kMfmaTileUs = 0.174;       // serial MFMA + LDS time per tile and 16-token block
-constexpr double kRoundUs = 3.61;           // start-up and drain of one round of workgroups
-constexpr double kNorm = 3.65;              // exponent that blends the three bounds
-constexpr double kCrowdPenalty = 0.072;     // per resident wave above kCrowdWaves on a unit
+constexpr double kCuBytesPerUs = 37.7e3;    // what one compute unit can pull on its own
+constexpr double kWaveTileUs = 0.649;       // a lone wave's turnaround per tile (latency bound)
+constexpr double kMfmaTileUs = 0.194;       // serial MFMA + LDS time per tile and 16-token block
+constexpr double kRoundUs = 4.61;           // start-up and drain of one round of workgroups
+constexpr double kNorm = 3.60;              // exponent that blends the three bounds
+constexpr double kCrowdPenalty = 0.048;     // per resident wave above kCrowdWaves on a unit
 constexpr double kCrowdWaves = 7.0;
-constexpr double kGlobalBPenalty = 0.154;   // mode 0, N <= 16, slice not staged
-constexpr double kModeKPenalty = 0.051;     // mode 1: activations from L2, reduction in LDS
-constexpr double kReduceUs = 3.14;          // fixed cost of the reduction kernel
-constexpr double kReduceBytesPerUs = 4.75e6;
+constexpr double kGlobalBPenalty = 0.0;   // mode 0, N <= 16, slice not staged
+constexpr double kModeKPenalty = 0.081;     // mode 1: activations from L2, reduction in LDS
+constexpr double kReduceUs = 4.02;          // fixed cost of the reduction as a second kernel (mode 0)
+constexpr double kFusedReduceUs = 2.28;     // ... and inside the main kernel (mode 1)
+constexpr double kReduceBytesPerUs = 5.42e6;
 
 int column_blocks(int N)
 {
@@ -142,7 +143,7 @@ double plan_cost_us(int M, int N, int K, int split_k, const LaunchPlan& p)
     if (p.mode == 1)
         total *= 1.0 + kModeKPenalty;
     if (split_k > 1)
-        total += kReduceUs + (2.0 * split_k + 1.0) * M * N * 2.0 / kReduceBytesPerUs;
+        total += (p.mode == 1 ? kFusedReduceUs : kReduceUs) + (2.0 * split_k + 1.0) * M * N * 2.0 / kReduceBytesPerUs;
     return total;
 }
 

@@ -110,12 +110,11 @@ int launch_main(void* stream, const void* Compressed_A, const int* TileOffsets, 
 {
     const tcsl::LaunchPlan p = o.forced ? *o.forced : cached_plan(M, N, K, Split_K, o.row_major);
     int page = -1;
-    if (fused_out) {
-        const long row_tiles = M / tcsl::kTileRows;
-        const long groups = p.mode ? row_tiles : (row_tiles + p.waves - 1) / p.waves;
-        if (groups <= 4096)
-            page = counter_page(stream);
-    }
+    // Only the layout whose workgroup owns a single tile row fuses the reduction: its last arriver
+    // adds up 128 rows.  In the row-sharing layout one workgroup would be left with W x 128 rows of
+    // every slab while the rest of the chip idles, which measured slower than the second kernel.
+    if (fused_out && p.mode == 1 && M / tcsl::kTileRows <= 4096)
+        page = counter_page(stream);
     if (fused)
         *fused = page >= 0;
     return tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, out, M, N, K, Split_K, p.mode, p.waves, p.stage_b,
@@ -163,12 +162,15 @@ extern "C" int SpMM_SplitK_API_Strided(void* stream, const void* Compressed_A, c
 
 extern "C" int SpMM_SplitK_API_Planned(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
                                        void* C, int M, int N, int K, void* Reduction_Workspace, int Split_K, int Mode,
-                                       int Waves, int StageB, int RowMajor)
+                                       int Waves, int StageB, int RowMajor, int Flags)
 {
     tcsl::LaunchPlan p{Mode, Waves, StageB, 0};
-    if (!tcsl::complete_plan(N, K > 0 ? K : 64, Split_K, RowMajor != 0, p))
+    if (!tcsl::complete_plan(N, K > 0 ? K : 64, Split_K, RowMajor != 0, p) ||
+        (Flags & ~(SPMM_FLAG_RELU | SPMM_FLAG_SEPARATE_REDUCTION)) != 0 || (RowMajor && (Flags & SPMM_FLAG_RELU)))
         return tcsl_error_invalid_value();
     CallOptions o;
+    o.relu = (Flags & SPMM_FLAG_RELU) != 0;
+    o.separate_reduction = (Flags & SPMM_FLAG_SEPARATE_REDUCTION) != 0;
     o.row_major = RowMajor != 0;
     o.forced = &p;
     return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, o);

@@ -115,33 +115,28 @@ __device__ __forceinline__ half8 load_activations_at(const _Float16* base, uint3
 // Stores and loads at system scope (write through every cache level / served from memory):
 // how the slabs of partial sums travel between workgroups of one launch without cache
 // maintenance.  A device-wide fence would write back and invalidate the whole L2 of the XCD,
-// which the weight stream lives in.
-__device__ __forceinline__ void store_through(_Float16* p, half8 v)
-{
-    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
-}
+// which the weight stream lives in.  Relaxed 64-bit atomics rather than inline assembly: the
+// compiler then also keeps the store data registers untouched for as long as the hardware
+// needs them (an assembly store's data was seen overwritten by the next VALU instruction).
 __device__ __forceinline__ void store_through(_Float16* p, half4 v)
 {
-    asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+    __hip_atomic_store(reinterpret_cast<uint64_t*>(p), __builtin_bit_cast(uint64_t, v), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_SYSTEM);
 }
-// Four independent 16-byte loads from memory; all have arrived when this returns.
-__device__ __forceinline__ void load_through4(const _Float16* p0, const _Float16* p1, const _Float16* p2,
-                                              const _Float16* p3, half8 (&w)[4])
+__device__ __forceinline__ void store_through(_Float16* p, half8 v)
 {
-    asm volatile("global_load_dwordx4 %0, %4, off sc0 sc1\n"
-                 "global_load_dwordx4 %1, %5, off sc0 sc1\n"
-                 "global_load_dwordx4 %2, %6, off sc0 sc1\n"
-                 "global_load_dwordx4 %3, %7, off sc0 sc1\n"
-                 "s_waitcnt vmcnt(0)"
-                 : "=&v"(w[0]), "=&v"(w[1]), "=&v"(w[2]), "=&v"(w[3])
-                 : "v"(p0), "v"(p1), "v"(p2), "v"(p3)
-                 : "memory");
+    typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
+    const u64x2 w = __builtin_bit_cast(u64x2, v);
+    __hip_atomic_store(reinterpret_cast<uint64_t*>(p), w[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    __hip_atomic_store(reinterpret_cast<uint64_t*>(p) + 1, w[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 __device__ __forceinline__ half8 load_through(const _Float16* p)
 {
-    half8 w;
-    asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1\n s_waitcnt vmcnt(0)" : "=&v"(w) : "v"(p) : "memory");
-    return w;
+    typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
+    u64x2 w;
+    w[0] = __hip_atomic_load(reinterpret_cast<const uint64_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    w[1] = __hip_atomic_load(reinterpret_cast<const uint64_t*>(p) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    return __builtin_bit_cast(half8, w);
 }
 
 // Wait until at most N vector-memory loads are outstanding (they complete in order).
@@ -643,7 +638,8 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
     // Fused split-K reduction.  Every workgroup has just written its slab; the last of the Split_K
     // workgroups that share a group of rows adds the slabs up, in slab order like the separate
     // kernel (csrc/Reduction_Kernel.cuh:36-46), so both paths give the same bits.
-    wait_loads<0>();  // this workgroup's partial sums (written through) have reached memory before it is counted
+    // this workgroup's partial sums (written through) have reached memory before it is counted
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), on top of what the compiler tracks itself
     __syncthreads();
     unsigned int* const counter = &tcsl_arrivals[fuse_page][blockIdx.x % groups];
     unsigned int* const flag = reinterpret_cast<unsigned int*>(lds);
@@ -664,8 +660,9 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
         int sidx = 0;
         for (; sidx + 4 <= split_k; sidx += 4) {
             half8 w[4];
-            load_through4(w0 + (size_t)sidx * slab, w0 + (size_t)(sidx + 1) * slab, w0 + (size_t)(sidx + 2) * slab,
-                          w0 + (size_t)(sidx + 3) * slab, w);
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                w[u] = load_through(w0 + (size_t)(sidx + u) * slab);
 #pragma unroll
             for (int u = 0; u < 4; u++)
 #pragma unroll

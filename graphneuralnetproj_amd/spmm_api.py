@@ -106,7 +106,7 @@ def load_library():
     lib.SpMM_PlanLaunch.argtypes = [ctypes.c_int] * 4 + [_i32p] * 4 + [ctypes.POINTER(ctypes.c_double)]
     lib.SpMM_SplitK_API_Planned.restype = ctypes.c_int
     lib.SpMM_SplitK_API_Planned.argtypes = ([ctypes.c_void_p] * 5 + [ctypes.c_int] * 3 + [ctypes.c_void_p]
-                                            + [ctypes.c_int] * 5)
+                                            + [ctypes.c_int] * 6)
     lib.SpMM_SplitK_API_Strided.restype = ctypes.c_int
     lib.SpMM_SplitK_API_Strided.argtypes = ([ctypes.c_void_p] * 4 + [ctypes.c_long, ctypes.c_void_p, ctypes.c_long]
                                             + [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_int, ctypes.c_int])
@@ -256,14 +256,14 @@ def SpMM_PlanLaunch(M_Global, N_Global, K_Global, Split_K):
 
 
 def SpMM_SplitK_API_Planned(stream, Compressed_A, TileOffsets, B, C, M_Global, N_Global, K_Global,
-                            Reduction_Workspace, Split_K, Mode, Waves, StageB, RowMajor=0):
+                            Reduction_Workspace, Split_K, Mode, Waves, StageB, RowMajor=0, Flags=0):
     """SpMM_SplitK_API with a caller-chosen launch shape (tuning and tests)."""
     lib = load_library()
     if stream is not None and not isinstance(stream, int):
         stream = stream.cuda_stream
     rc = lib.SpMM_SplitK_API_Planned(ctypes.c_void_p(stream) if stream else None, _ptr(Compressed_A), _ptr(TileOffsets),
                                      _ptr(B), _ptr(C), M_Global, N_Global, K_Global, _ptr(Reduction_Workspace),
-                                     Split_K, Mode, Waves, StageB, RowMajor)
+                                     Split_K, Mode, Waves, StageB, RowMajor, Flags)
     if rc != 0:
         raise SpMMError("SpMM_SplitK_API_Planned", rc, lib.SpMM_GetErrorString(rc).decode())
     return rc

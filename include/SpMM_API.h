@@ -63,7 +63,8 @@ SPMM_EXPORT int InitSparseMatrixA_API(const uint16_t* A_h, int M, int N, int K, 
  *   Split_K  > 1: batch b of ceil((K/64)/Split_K) column tiles writes fp16 partial
  *                 sums to Reduction_Workspace[b*M*N ..), then C = fp16(sum in fp32), added
  *                 up in batch order either by the last workgroup of the same launch to
- *                 finish a group of rows or by a second kernel (same bits either way).
+ *                 finish a tile row (launch shape "mode 1", M <= 524288) or by a second
+ *                 kernel (same bits either way).
  *                 Reduction_Workspace must hold Split_K*M*N fp16 values and may be
  *                 shared by successive calls on one stream.
  * Accumulation is fp32.  Returns the hipError_t value: 0 on success;
@@ -181,11 +182,12 @@ SPMM_EXPORT int SpMM_PlanLaunch(int M_Global, int N_Global, int K_Global, int Sp
  * (for tuning a table of plans on the target machine, and for tests).  Returns
  * hipErrorInvalidValue when the shape does not fit (Waves above 8, or 4 for N = 64;
  * StageB with Mode 1, N > 16 or RowMajor; more than 160 KiB of LDS).  RowMajor != 0 selects
- * the operand layout of SpMM_SplitK_API_RowMajor.  No counterpart in the reference.
+ * the operand layout of SpMM_SplitK_API_RowMajor; Flags as for SpMM_SplitK_API_Strided (no
+ * clamp with row-major operands).  No counterpart in the reference.
  */
 SPMM_EXPORT int SpMM_SplitK_API_Planned(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
                                         void* C, int M_Global, int N_Global, int K_Global, void* Reduction_Workspace,
-                                        int Split_K, int Mode, int Waves, int StageB, int RowMajor);
+                                        int Split_K, int Mode, int Waves, int StageB, int RowMajor, int Flags);
 
 /*
  * Deterministic synthetic inputs for tests and benchmarks (host memory, fp16 bit

@@ -525,3 +525,29 @@ def test_fused_reduction_on_two_streams(spmm, oracle):
     torch.cuda.synchronize()
     for (ref, _, _, _, c, _, _) in cases:
         assert_close(c.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("N,split_k,mode,waves,stage_b", [
+    (32, 8, 0, 1, 0),   # one-wave workgroups, eight resident per compute unit: hundreds finish together
+    (16, 8, 0, 7, 1), (16, 4, 1, 6, 0), (64, 4, 0, 4, 0), (8, 6, 1, 8, 0),
+])
+def test_fused_reduction_under_load_bit_for_bit(spmm, N, split_k, mode, waves, stage_b):
+    """Full-size weight: every compute unit busy and many workgroups arriving at once."""
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    M, K = 28672, 7168
+    A, B, items, offsets = make_case(spmm, M, K, N, 0.8, seed=4242)
+    d_items = torch.from_numpy(items.view(np.int32).copy()).to(dev)
+    d_offs = torch.from_numpy(offsets.copy()).to(dev)
+    d_B = torch.from_numpy(np.ascontiguousarray(B).view(np.int16).copy()).to(dev)
+    outs = []
+    for flags in (spmm.SPMM_FLAG_SEPARATE_REDUCTION, 0, 0, 0):
+        d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device=dev)
+        d_W = torch.full((split_k, N, M), float("nan"), dtype=torch.float16, device=dev)
+        print(f"[gpu case] fused under load N={N} split_k={split_k} plan=({mode},{waves},{stage_b}) flags={flags}", flush=True)
+        spmm.SpMM_SplitK_API_Planned(torch.cuda.current_stream(), d_items, d_offs, d_B, d_C, M, N, K, d_W, split_k,
+                                     mode, waves, stage_b, 0, flags)
+        torch.cuda.synchronize()
+        outs.append(d_C.cpu().numpy().view(np.uint16))
+    for o in outs[1:]:
+        assert np.array_equal(outs[0], o)
