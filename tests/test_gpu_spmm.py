@@ -446,9 +446,15 @@ def test_decoder_stack_matches_cpu_chain(spmm, oracle):
         f = f16(np.maximum(oracle.gemm_f32(d["ffn1"], o), 0.0))
         x = f16(oracle.gemm_f32(d["ffn2"], f))
     assert np.abs(x.astype(np.float32)).max() > 1e-3, "the reference chain must not have collapsed to zero"
-    # each product is within the per-call tolerance; four roundings per layer compound, so allow 3x
-    err = np.abs(got.astype(np.float32) - x.astype(np.float32))
-    assert (err <= 3 * (ATOL + RTOL * np.abs(x.astype(np.float32)))).all(), err.max()
+    # Each product is within the per-call tolerance of its own inputs, but the inputs of later
+    # products already differ by the earlier roundings (fp16 storage of every intermediate, and
+    # split-K partial sums on the GPU only), and an output element near zero is a sum of large
+    # terms that cancel: its error scales with the typical magnitude, not with its own.  So the
+    # per-element tolerance is taken against max(|ref|, rms(ref)), times 3 for the twelve products.
+    xr = x.astype(np.float32)
+    err = np.abs(got.astype(np.float32) - xr)
+    scale = np.maximum(np.abs(xr), np.sqrt(np.mean(xr * xr)))
+    assert (err <= 3 * (ATOL + RTOL * scale)).all(), err.max()
 
 
 @pytest.mark.parametrize("M,K,N,split_k", [
