@@ -421,12 +421,8 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
             return;  // empty tile or past the end
         static_for<VPL>([&](auto uc) {
             constexpr int u = decltype(uc)::value;
-            if (u * kWave < s.n) {
-                if ((u + 1) * kWave <= s.n)
-                    scatter_words<false>(regs[slot][u], vbase, vtwo, vzero);
-                else if (u * kWave + lane < s.n)  // the segment's last, partial chunk
-                    scatter_words<false>(regs[slot][u], vbase, vtwo, vzero);
-            }
+            if (__builtin_expect(u * kWave + lane < s.n, 1))  // lanes past the segment's end sit out
+                scatter_words<false>(regs[slot][u], vbase, vtwo, vzero);
         });
         if (!s.last)
             return;  // more segments of this tile follow
@@ -486,12 +482,8 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
         } else {
             static_for<VPL>([&](auto uc) {
                 constexpr int u = decltype(uc)::value;
-                if (u * kWave < s.n) {
-                    if ((u + 1) * kWave <= s.n)
-                        scatter_words<true>(regs[slot][u], vbase, vtwo, vzero);
-                    else if (u * kWave + lane < s.n)
-                        scatter_words<true>(regs[slot][u], vbase, vtwo, vzero);
-                }
+                if (__builtin_expect(u * kWave + lane < s.n, 1))
+                    scatter_words<true>(regs[slot][u], vbase, vtwo, vzero);
             });
         }
     };

@@ -86,7 +86,7 @@ def test_small_vs_oracle(spmm, oracle, N, split_k):
 
 
 def test_config1_cpu_reference_case(spmm, oracle):
-    """BASELINE config 1: M=K=1024, N=8, 80 % Bernoulli, Split_K=1, seed 0."""
+    """The CPU-runnable reference case: M=K=1024, N=8, 80 % Bernoulli, Split_K=1, seed 0."""
     M = K = 1024
     A, B, items, offsets = make_case(spmm, M, K, 8, 0.8, seed=0)
     C, _ = run_gpu(spmm, items, offsets, B, M, 8, K, 1)
