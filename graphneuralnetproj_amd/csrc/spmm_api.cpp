@@ -16,6 +16,8 @@ int tcsl_launch_spmm(void* stream, const void* items, const int* offsets, const 
                      int ldo, int relu, void* fused_out, int ldc, int fuse_page);
 int tcsl_launch_reduce(void* stream, void* C, const void* W, long rows, long vectors, long ldc, int split_k, int relu);
 int tcsl_launch_copy(void* stream, void* dst, const void* src, long bytes);
+int tcsl_launch_encode_offsets(void* stream, const void* A, int M, int K, int* offsets);
+int tcsl_launch_encode_items(void* stream, const void* A, int M, int K, const int* offsets, void* items);
 void* tcsl_event_create(void);
 void tcsl_event_destroy(void* e);
 int tcsl_event_record(void* e, void* stream);
@@ -36,6 +38,22 @@ extern "C" int GenSparseMatrixBinFile(char* DenseMatrixFileName, int M, int K, c
                                       char* TileOffsetsFileName, char* OutputSizesFileName)
 {
     return tcsl::encode_file(DenseMatrixFileName, M, K, NZWeightsFileName, TileOffsetsFileName, OutputSizesFileName);
+}
+
+extern "C" int SpMM_DeviceEncodeOffsets(void* stream, const void* A_d, int M, int K, int* TileOffsets_d)
+{
+    if (M <= 0 || K <= 0 || M % tcsl::kTileRows != 0 || K % tcsl::kTileCols != 0 || !A_d || !TileOffsets_d)
+        return tcsl_error_invalid_value();
+    return tcsl_launch_encode_offsets(stream, A_d, M, K, TileOffsets_d);
+}
+
+extern "C" int SpMM_DeviceEncodeItems(void* stream, const void* A_d, int M, int K, const int* TileOffsets_d,
+                                      void* Compressed_A_d)
+{
+    if (M <= 0 || K <= 0 || M % tcsl::kTileRows != 0 || K % tcsl::kTileCols != 0 || !A_d || !TileOffsets_d ||
+        !Compressed_A_d)
+        return tcsl_error_invalid_value();
+    return tcsl_launch_encode_items(stream, A_d, M, K, TileOffsets_d, Compressed_A_d);
 }
 
 extern "C" void SpMM_FreeHost(void* p)

@@ -35,6 +35,8 @@ EXPORTED_SYMBOLS = (
     "SpMM_SplitK_API_Planned",
     "SpMM_SplitK_API_RowMajor",
     "SpMM_SplitK_API_Strided",
+    "SpMM_DeviceEncodeOffsets",
+    "SpMM_DeviceEncodeItems",
     "SpMM_SynthWeights",
     "SpMM_SynthActivations",
     "SpMM_CalibrationCopy",
@@ -110,6 +112,11 @@ def load_library():
     lib.SpMM_SplitK_API_Strided.restype = ctypes.c_int
     lib.SpMM_SplitK_API_Strided.argtypes = ([ctypes.c_void_p] * 4 + [ctypes.c_long, ctypes.c_void_p, ctypes.c_long]
                                             + [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_int, ctypes.c_int])
+    lib.SpMM_DeviceEncodeOffsets.restype = ctypes.c_int
+    lib.SpMM_DeviceEncodeOffsets.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    lib.SpMM_DeviceEncodeItems.restype = ctypes.c_int
+    lib.SpMM_DeviceEncodeItems.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                           ctypes.c_void_p]
     lib.SpMM_SplitK_API_RowMajor.restype = ctypes.c_int
     lib.SpMM_SplitK_API_RowMajor.argtypes = lib.SpMM_SplitK_API.argtypes
     lib.SpMM_SynthWeights.restype = None
@@ -228,6 +235,35 @@ def SpMM_SplitK_API_Strided(stream, Compressed_A, TileOffsets, B, ldb, C, ldc, M
     if rc != 0:
         raise SpMMError("SpMM_SplitK_API_Strided", rc, lib.SpMM_GetErrorString(rc).decode())
     return rc
+
+
+def encode_on_device(A_d, stream=None):
+    """Tiled-CSL encode of a torch CUDA fp16 matrix on the GPU -> (items int32 tensor, offsets int32 tensor).
+
+    Same bits as InitSparseMatrixA_API; synchronises once to size the word buffer.
+    """
+    import torch
+
+    lib = load_library()
+    M, K = A_d.shape
+    if A_d.dtype != torch.float16 or not A_d.is_contiguous():
+        raise TypeError("expected a contiguous float16 CUDA tensor")
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    sptr = ctypes.c_void_p(stream.cuda_stream) if stream.cuda_stream else None
+    tiles = (M // 128) * (K // 64)
+    offsets = torch.empty(max(tiles, 0) + 2, dtype=torch.int32, device=A_d.device)
+    rc = lib.SpMM_DeviceEncodeOffsets(sptr, _ptr(A_d), M, K, _ptr(offsets))
+    if rc != 0:
+        raise SpMMError("SpMM_DeviceEncodeOffsets", rc, lib.SpMM_GetErrorString(rc).decode())
+    vectors = int(offsets[-1].item())  # synchronises
+    if vectors < 0:
+        raise SpMMError("SpMM_DeviceEncodeOffsets", -5, "more than 2^31-1 vectors")
+    items = torch.empty(max(vectors * 4, 4), dtype=torch.int32, device=A_d.device)
+    rc = lib.SpMM_DeviceEncodeItems(sptr, _ptr(A_d), M, K, _ptr(offsets), _ptr(items))
+    if rc != 0:
+        raise SpMMError("SpMM_DeviceEncodeItems", rc, lib.SpMM_GetErrorString(rc).decode())
+    return items[: vectors * 4], offsets
 
 
 def GenSparseMatrixBinFile(DenseMatrixFileName, M, K, NZWeightsFileName, TileOffsetsFileName, OutputSizesFileName):

@@ -149,6 +149,23 @@ SPMM_EXPORT float SpMM_EventElapsedMs(void* start, void* stop);
 SPMM_EXPORT int GenSparseMatrixBinFile(char* DenseMatrixFileName, int M, int K, char* NZWeightsFileName,
                            char* TileOffsetsFileName, char* OutputSizesFileName);
 
+/*
+ * The encoder on the GPU, for weights that are already in device memory (row-major M x K
+ * fp16 at A_d): same bits as InitSparseMatrixA_API.  Two steps, because the caller owns
+ * the output buffers and their size depends on the data:
+ *   SpMM_DeviceEncodeOffsets  fills TileOffsets_d ((M/128)*(K/64) + 2 ints);
+ *                             the last entry, V, is the number of 16-byte vectors
+ *                             (-1 if it would not fit an int);
+ *   SpMM_DeviceEncodeItems    fills Compressed_A_d (16 * V bytes) from A_d and those offsets.
+ * Both only enqueue kernels on `stream`; read V back (after synchronising) to size the
+ * second buffer, or allocate the worst case M*K*4 + 16*tiles bytes up front.  Return a
+ * hipError_t value; hipErrorInvalidValue for M % 128, K % 64 or null pointers.  The
+ * reference encodes on one host thread only (csrc/SpMM_API.cu:241-438).
+ */
+SPMM_EXPORT int SpMM_DeviceEncodeOffsets(void* stream, const void* A_d, int M, int K, int* TileOffsets_d);
+SPMM_EXPORT int SpMM_DeviceEncodeItems(void* stream, const void* A_d, int M, int K, const int* TileOffsets_d,
+                                       void* Compressed_A_d);
+
 /* free() for buffers returned by InitSparseMatrixA_API (for callers without a C runtime at hand). */
 SPMM_EXPORT void SpMM_FreeHost(void* p);
 
