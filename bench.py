@@ -119,6 +119,8 @@ def main():
     ap.add_argument("--skew", action="store_true")
     ap.add_argument("--split-k", type=int, default=0, help="0 = SpMM_SuggestSplitK")
     ap.add_argument("--copies", type=int, default=0, help="distinct HBM copies of the weight (0 = enough for > 640 MB)")
+    ap.add_argument("--no-reorder", action="store_true",
+                    help="encode with InitSparseMatrixA_API_NoReorder (the reference's ablation of its bank-aware reordering)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
     ap.add_argument("--calibration-copies", type=int, default=0,
@@ -155,7 +157,7 @@ def main():
     B = G.synth_activations(N, K, seed=4321)
     t_synth = time.perf_counter() - t0
     t0 = time.perf_counter()
-    items, offsets = G.InitSparseMatrixA_API(A)
+    items, offsets = (G.InitSparseMatrixA_API_NoReorder if args.no_reorder else G.InitSparseMatrixA_API)(A)
     t_encode = time.perf_counter() - t0
     a_bytes = 16 * int(offsets[-1])
     copies = args.copies or max(2, -(-640 * 1024 * 1024 // max(a_bytes, 1)))
@@ -260,6 +262,7 @@ def main():
                                         + (4 * split_k * M * N if split_k > 1 else 0)),
             "weight_copies_rotated": copies,
             "layout": "B[N][K], C[N][M]",
+            "encoding": "scan order (no reordering)" if args.no_reorder else "bank-aware reordering",
         },
         "hbm_gbps": a_bytes / (ms_per_step * 1e-3) / 1e9,
         "hbm_frac_of_peak": a_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,

@@ -34,6 +34,13 @@ extern "C" int InitSparseMatrixA_API(const uint16_t* A_h, int M, int N, int K, u
     return tcsl::encode(A_h, M, K, Compressed_A, TileOffsets);
 }
 
+extern "C" int InitSparseMatrixA_API_NoReorder(const uint16_t* A_h, int M, int N, int K, uint32_t** Compressed_A,
+                                               int** TileOffsets)
+{
+    (void)N;
+    return tcsl::encode_noreorder(A_h, M, K, Compressed_A, TileOffsets);
+}
+
 extern "C" int GenSparseMatrixBinFile(char* DenseMatrixFileName, int M, int K, char* NZWeightsFileName,
                                       char* TileOffsetsFileName, char* OutputSizesFileName)
 {

@@ -165,9 +165,44 @@ int emit_tile(const uint16_t* tile, int ld, uint32_t* dst, TileScratch& ws)
     return count;
 }
 
+// One tile without reordering (csrc/SpMM_API.cu:514-551): kept elements in scan order, and the
+// first `pads` elements of the scan that are not kept, with whatever bits they hold.
+int emit_tile_noreorder(const uint16_t* tile, int ld, uint32_t* dst, int pads)
+{
+    int w = 0;
+    for (int m = 0; m < kTileRows; m++) {
+        const uint16_t* row = tile + static_cast<size_t>(m) * ld;
+        const int flip = (m & 7) << 3;
+        for (int n = 0; n < kTileCols; n++) {
+            const uint16_t v = row[n];
+            if (kept(v)) {
+                dst[w++] = pack_item(v, m * kTileCols + (n ^ flip));
+            } else if (pads > 0) {
+                pads--;
+                dst[w++] = pack_item(v, m * kTileCols + (n ^ flip));
+            }
+        }
+    }
+    return w;
+}
+
+int encode_impl(const uint16_t* A, int M, int K, uint32_t** items_out, int** offsets_out, bool reorder);
+
 }  // namespace
 
 int encode(const uint16_t* A, int M, int K, uint32_t** items_out, int** offsets_out)
+{
+    return encode_impl(A, M, K, items_out, offsets_out, true);
+}
+
+int encode_noreorder(const uint16_t* A, int M, int K, uint32_t** items_out, int** offsets_out)
+{
+    return encode_impl(A, M, K, items_out, offsets_out, false);
+}
+
+namespace {
+
+int encode_impl(const uint16_t* A, int M, int K, uint32_t** items_out, int** offsets_out, bool reorder)
 {
     if (!A || !items_out || !offsets_out)
         return kErrNullPointer;
@@ -215,8 +250,15 @@ int encode(const uint16_t* A, int M, int K, uint32_t** items_out, int** offsets_
         }
         for (int j = 0; j < tc; j++) {
             const long t = i * tc + j;
-            const int n = emit_tile(A + static_cast<size_t>(i) * kTileRows * K + static_cast<size_t>(j) * kTileCols, K,
-                                    items + static_cast<size_t>(offs[t]) * kVec, *ws);
+            const uint16_t* tile = A + static_cast<size_t>(i) * kTileRows * K + static_cast<size_t>(j) * kTileCols;
+            uint32_t* dst = items + static_cast<size_t>(offs[t]) * kVec;
+            int n;
+            if (reorder) {
+                n = emit_tile(tile, K, dst, *ws);
+            } else {
+                const int nz = count_tile(tile, K);
+                n = emit_tile_noreorder(tile, K, dst, (kVec - nz % kVec) % kVec);
+            }
             if (n != (offs[t + 1] - offs[t]) * kVec)
                 ok = false;
         }
@@ -231,6 +273,8 @@ int encode(const uint16_t* A, int M, int K, uint32_t** items_out, int** offsets_
     *offsets_out = offs;
     return static_cast<int>(ntiles + kOffsetPadding);
 }
+
+}  // namespace
 
 int encode_file(const char* dense, int M, int K, const char* nz_path, const char* off_path, const char* sizes_path)
 {

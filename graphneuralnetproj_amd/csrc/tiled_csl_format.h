@@ -28,6 +28,7 @@ inline uint32_t pack_item(uint16_t value_bits, int position)
 }
 
 int encode(const uint16_t* A, int M, int K, uint32_t** items_out, int** offsets_out);
+int encode_noreorder(const uint16_t* A, int M, int K, uint32_t** items_out, int** offsets_out);
 int encode_file(const char* dense, int M, int K, const char* nz_path, const char* off_path, const char* sizes_path);
 
 // Deterministic synthetic inputs (counter based, identical on every host).

@@ -26,6 +26,7 @@ _i32p = ctypes.POINTER(ctypes.c_int)
 
 EXPORTED_SYMBOLS = (
     "InitSparseMatrixA_API",
+    "InitSparseMatrixA_API_NoReorder",
     "SpMM_SplitK_API",
     "GenSparseMatrixBinFile",
     "SpMM_FreeHost",
@@ -93,6 +94,8 @@ def load_library():
     lib.InitSparseMatrixA_API.restype = ctypes.c_int
     lib.InitSparseMatrixA_API.argtypes = [_u16p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(_u32p),
                                           ctypes.POINTER(_i32p)]
+    lib.InitSparseMatrixA_API_NoReorder.restype = ctypes.c_int
+    lib.InitSparseMatrixA_API_NoReorder.argtypes = lib.InitSparseMatrixA_API.argtypes
     lib.SpMM_SplitK_API.restype = ctypes.c_int
     lib.SpMM_SplitK_API.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_int]
     lib.GenSparseMatrixBinFile.restype = ctypes.c_int
@@ -151,7 +154,12 @@ def _bits(a):
     return a
 
 
-def InitSparseMatrixA_API(A_h, M=None, N=0, K=None):
+def InitSparseMatrixA_API_NoReorder(A_h, M=None, N=0, K=None):
+    """InitSparseMatrixA_API without the bank-aware reordering of a tile's words."""
+    return InitSparseMatrixA_API(A_h, M, N, K, _entry="InitSparseMatrixA_API_NoReorder")
+
+
+def InitSparseMatrixA_API(A_h, M=None, N=0, K=None, _entry="InitSparseMatrixA_API"):
     """Encode a row-major fp16 M x K host matrix.
 
     Returns (Compressed_A uint32[4*TileOffsets[-1]], TileOffsets int32[(M/128)*(K/64)+2]);
@@ -165,9 +173,9 @@ def InitSparseMatrixA_API(A_h, M=None, N=0, K=None):
         raise ValueError(f"A_h has {a.size} elements, expected {M}*{K}")
     lib = load_library()
     items, offs = _u32p(), _i32p()
-    n = lib.InitSparseMatrixA_API(a.ctypes.data_as(_u16p), M, N, K, ctypes.byref(items), ctypes.byref(offs))
+    n = getattr(lib, _entry)(a.ctypes.data_as(_u16p), M, N, K, ctypes.byref(items), ctypes.byref(offs))
     if n < 0:
-        raise SpMMError("InitSparseMatrixA_API", n)
+        raise SpMMError(_entry, n)
     offsets = np.ctypeslib.as_array(offs, shape=(n,)).astype(np.int32, copy=True)
     nwords = int(offsets[-1]) * 4
     compressed = (np.ctypeslib.as_array(items, shape=(nwords,)).astype(np.uint32, copy=True)

@@ -48,6 +48,20 @@ extern "C" {
 SPMM_EXPORT int InitSparseMatrixA_API(const uint16_t* A_h, int M, int N, int K, uint32_t** Compressed_A, int** TileOffsets);
 
 /*
+ * The encoder without its bank-aware reordering.  Stands in for
+ *   int InitSparseMatrixA_API_NoReorder(half* A_h, int M, int N, int K, uint32_t** Compressed_A, int** TileOffsets)
+ *   (declared build/SpMM_API.cuh:57-62, defined csrc/SpMM_API.cu:441-567), the reference's
+ *   ablation of "ahead of time sparse data reordering".
+ * Same conventions and return codes as InitSparseMatrixA_API, same TileOffsets; the words of a
+ * tile come in scan order.  Bit-identical to the reference's, including that a padding word
+ * carries the bits of the element it points at (+0 normally, but -0 or a NaN pattern if that is
+ * what the matrix holds there).  Every SpMM entry point accepts either encoding: a word carries
+ * its own position.
+ */
+SPMM_EXPORT int InitSparseMatrixA_API_NoReorder(const uint16_t* A_h, int M, int N, int K, uint32_t** Compressed_A,
+                                                int** TileOffsets);
+
+/*
  * The product C = A * B on the GPU.  Stands in for
  *   cudaError_t SpMM_SplitK_API(cudaStream_t stream, const half* A, const uint4* Compressed_A,
  *                               const int* TileOffsets, const half* B, half* C,

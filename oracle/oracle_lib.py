@@ -38,6 +38,8 @@ def _load():
     lib.oracle_float_to_half_rn.argtypes = [ctypes.c_float]
     lib.oracle_encode.restype = ctypes.c_int
     lib.oracle_encode.argtypes = [_u16p, ctypes.c_int, ctypes.c_int, ctypes.POINTER(_u32p), ctypes.POINTER(_i32p)]
+    lib.oracle_encode_noreorder.restype = ctypes.c_int
+    lib.oracle_encode_noreorder.argtypes = lib.oracle_encode.argtypes
     lib.oracle_free.argtypes = [ctypes.c_void_p]
     lib.oracle_decode.argtypes = [_u32p, _i32p, ctypes.c_int, ctypes.c_int, _u16p]
     lib.oracle_gemm_f32.argtypes = [_u16p, _u16p, _f32p] + [ctypes.c_int] * 5
@@ -82,6 +84,20 @@ def encode(A):
     n = lib().oracle_encode(a.ctypes.data_as(_u16p), M, K, ctypes.byref(items), ctypes.byref(offs))
     if n < 0:
         raise ValueError(f"oracle_encode failed with {n} for M={M} K={K}")
+    o = np.ctypeslib.as_array(offs, shape=(n,)).astype(np.int32, copy=True)
+    it = _take(items, int(o[-1]) * 4, np.uint32, lib().oracle_free)
+    lib().oracle_free(offs)
+    return it, o
+
+
+def encode_noreorder(A):
+    """Oracle encode without the bank-aware reordering (csrc/SpMM_API.cu:441-567)."""
+    M, K = A.shape
+    a = _bits(A)
+    items, offs = _u32p(), _i32p()
+    n = lib().oracle_encode_noreorder(a.ctypes.data_as(_u16p), M, K, ctypes.byref(items), ctypes.byref(offs))
+    if n < 0:
+        raise ValueError(f"oracle_encode_noreorder failed with {n} for M={M} K={K}")
     o = np.ctypeslib.as_array(offs, shape=(n,)).astype(np.int32, copy=True)
     it = _take(items, int(o[-1]) * 4, np.uint32, lib().oracle_free)
     lib().oracle_free(offs)
@@ -146,19 +162,23 @@ def have_ref():
 _ref = None
 
 
-def ref_encode(A):
-    """Encode with the reference's InitSparseMatrixA_API (csrc/SpMM_API.cu:241-438)."""
+def ref_encode(A, reorder=True):
+    """Encode with the reference's InitSparseMatrixA_API (csrc/SpMM_API.cu:241-438) or, with
+    reorder=False, its InitSparseMatrixA_API_NoReorder (:441-567)."""
     global _ref
     if _ref is None:
         _ref = ctypes.CDLL(_REF_SO)
         _ref.ref_InitSparseMatrixA_API.restype = ctypes.c_int
         _ref.ref_InitSparseMatrixA_API.argtypes = [_u16p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                    ctypes.POINTER(_u32p), ctypes.POINTER(_i32p)]
+        _ref.ref_InitSparseMatrixA_API_NoReorder.restype = ctypes.c_int
+        _ref.ref_InitSparseMatrixA_API_NoReorder.argtypes = _ref.ref_InitSparseMatrixA_API.argtypes
         _ref.ref_free.argtypes = [ctypes.c_void_p]
     M, K = A.shape
     a = _bits(A).copy()
     items, offs = _u32p(), _i32p()
-    n = _ref.ref_InitSparseMatrixA_API(a.ctypes.data_as(_u16p), M, 0, K, ctypes.byref(items), ctypes.byref(offs))
+    fn = _ref.ref_InitSparseMatrixA_API if reorder else _ref.ref_InitSparseMatrixA_API_NoReorder
+    n = fn(a.ctypes.data_as(_u16p), M, 0, K, ctypes.byref(items), ctypes.byref(offs))
     o = np.ctypeslib.as_array(offs, shape=(n,)).astype(np.int32, copy=True)
     it = _take(items, int(o[-1]) * 4, np.uint32, _ref.ref_free)
     _ref.ref_free(offs)

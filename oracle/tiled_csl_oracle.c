@@ -12,6 +12,10 @@
  *                          compiled from csrc/SpMM_API.cu:210-438 (oracle/_ref)
  *                          and with committed golden vectors made by it;
  *                          hand-derived micro cases; format invariants.
+ *   oracle_encode_noreorder - bit-compared with the reference's own
+ *                          InitSparseMatrixA_API_NoReorder compiled from
+ *                          csrc/SpMM_API.cu:441-567 (oracle/_ref) and with committed
+ *                          golden vectors made by it; decode(encode) == A.
  *   oracle_decode        - closed-form inverse of the index packing
  *                          (csrc/SpMM_API.cu:330-339); decode(encode(A)) == A.
  *   oracle_gemm_f32      - textbook fp32-accumulate product; checked against
@@ -263,6 +267,62 @@ int oracle_encode(const uint16_t *A, int M, int K, uint32_t **items, int **offse
         free(offs);
         return -4;
     }
+    *items = out;
+    *offsets = offs;
+    return (int)(ntiles + 2);
+}
+
+/* Tiled-CSL encode without the bank-aware reordering (csrc/SpMM_API.cu:441-567): the kept
+ * elements of a tile in scan order, and, interleaved with them, the first `pad` elements of
+ * the scan that are not kept, carrying their own bits as the value (:533-546; normally +0,
+ * but -0 and NaN bit patterns are copied as they are).  Same return convention as
+ * oracle_encode. */
+int oracle_encode_noreorder(const uint16_t *A, int M, int K, uint32_t **items, int **offsets)
+{
+    if (M <= 0 || K <= 0 || M % ORACLE_TILE_ROWS || K % ORACLE_TILE_COLS)
+        return -1;
+    const int tr = M / ORACLE_TILE_ROWS, tc = K / ORACLE_TILE_COLS;
+    const long ntiles = (long)tr * tc;
+    long total = 0;
+    for (int i = 0; i < tr; i++)
+        for (int j = 0; j < tc; j++) {
+            int nz = 0;
+            for (int m = 0; m < ORACLE_TILE_ROWS; m++)
+                for (int n = 0; n < ORACLE_TILE_COLS; n++)
+                    nz += is_kept(A[(size_t)(i * ORACLE_TILE_ROWS + m) * K + j * ORACLE_TILE_COLS + n]);
+            total += nz + (ORACLE_VEC - nz % ORACLE_VEC) % ORACLE_VEC;
+        }
+    uint32_t *out = (uint32_t *)malloc((total ? total : 1) * sizeof(uint32_t));
+    int *offs = (int *)malloc((ntiles + 2) * sizeof(int));
+    if (!out || !offs) {
+        free(out);
+        free(offs);
+        return -2;
+    }
+    long w = 0;
+    for (int i = 0; i < tr; i++)
+        for (int j = 0; j < tc; j++) {
+            const uint16_t *tile = A + (size_t)i * ORACLE_TILE_ROWS * K + (size_t)j * ORACLE_TILE_COLS;
+            int nz = 0;
+            for (int m = 0; m < ORACLE_TILE_ROWS; m++)
+                for (int n = 0; n < ORACLE_TILE_COLS; n++)
+                    nz += is_kept(tile[(size_t)m * K + n]);
+            int pads = (ORACLE_VEC - nz % ORACLE_VEC) % ORACLE_VEC;
+            for (int m = 0; m < ORACLE_TILE_ROWS; m++)
+                for (int n = 0; n < ORACLE_TILE_COLS; n++) {
+                    const uint16_t v = tile[(size_t)m * K + n];
+                    const uint32_t pos = (uint32_t)(m * ORACLE_TILE_COLS + (n ^ ((m % 8) << 3)));
+                    if (is_kept(v)) {
+                        out[w++] = (uint32_t)v | pos << 16;
+                    } else if (pads > 0) {
+                        pads--;
+                        out[w++] = (uint32_t)v | pos << 16;
+                    }
+                }
+            offs[(long)i * tc + j + 1] = (int)(w / ORACLE_VEC);
+        }
+    offs[0] = 0;
+    offs[ntiles + 1] = (int)(w / ORACLE_VEC);
     *items = out;
     *offsets = offs;
     return (int)(ntiles + 2);

@@ -557,3 +557,14 @@ def test_fused_reduction_under_load_bit_for_bit(spmm, N, split_k, mode, waves, s
         outs.append(d_C.cpu().numpy().view(np.uint16))
     for o in outs[1:]:
         assert np.array_equal(outs[0], o)
+
+
+@pytest.mark.parametrize("N,split_k", [(16, 1), (8, 3), (64, 2)])
+def test_product_on_unreordered_encoding(spmm, oracle, N, split_k):
+    """The kernels take a tile's words in any order: the reference's no-reorder encoding works unchanged."""
+    M, K = 512, 1024
+    A = spmm.synth_weights(M, K, 0.8, False, seed=31 + N)
+    B = spmm.synth_activations(N, K, seed=32)
+    items, offsets = spmm.InitSparseMatrixA_API_NoReorder(A)
+    C, _ = run_gpu(spmm, items, offsets, B, M, N, K, split_k)
+    assert_close(C, oracle.gemm_f32(A, B))

@@ -178,3 +178,25 @@ def test_planner_uses_every_compute_unit_on_the_headline_shapes(spmm):
         p = spmm.SpMM_PlanLaunch(M, 16, K, s)
         wgs = (M // 128) * s if p["mode"] == 1 else -(-(M // 128) // p["waves"]) * s
         assert 200 <= wgs <= 512, (M, K, s, p)
+
+
+def test_noreorder_encoder_matches_golden_and_oracle(spmm, oracle):
+    z = np.load(os.path.join(GOLD, "encoder_small.npz"))
+    names = sorted({k.rsplit(".", 1)[0] for k in z.files})
+    for n in names:
+        items, offs = spmm.InitSparseMatrixA_API_NoReorder(z[n + ".A"])
+        assert np.array_equal(offs, z[n + ".offsets"]), n
+        assert np.array_equal(items, z[n + ".items_noreorder"]), n
+    with open(os.path.join(GOLD, "encoder_large.json")) as f:
+        cases = json.load(f)
+    for c in cases:
+        A = spmm.synth_weights(c["M"], c["K"], c["sparsity"], c["row_skewed"], seed=c["seed"])
+        items, offs = spmm.InitSparseMatrixA_API_NoReorder(A)
+        assert hashlib.sha256(items.tobytes()).hexdigest() == c["items_noreorder_sha256"]
+        assert hashlib.sha256(offs.tobytes()).hexdigest() == c["offsets_sha256"]
+    A = spmm.synth_weights(640, 448, 0.75, True, seed=9)
+    items, offs = spmm.InitSparseMatrixA_API_NoReorder(A)
+    o_items, o_offs = oracle.encode_noreorder(A)
+    assert np.array_equal(items, o_items) and np.array_equal(offs, o_offs)
+    with pytest.raises(spmm.SpMMError):
+        spmm.InitSparseMatrixA_API_NoReorder(np.zeros((100, 64), dtype=np.float16))

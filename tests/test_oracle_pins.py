@@ -249,3 +249,49 @@ def test_spmm_splitk_slabs_sum_to_full_product(oracle):
             s, e = oracle.splitk_range(K, split_k, 1)
             part = B[:, s * 64:e * 64].astype(np.float64) @ A[:, s * 64:e * 64].astype(np.float64).T
             assert np.array_equal(W[1].astype(np.float64), part)
+
+
+# ------------------------------------------------- encoder, no reordering ---
+
+def test_noreorder_encode_matches_reference_golden(oracle, spmm):
+    import hashlib
+
+    z = np.load(os.path.join(GOLD, "encoder_small.npz"))
+    names = sorted({k.rsplit(".", 1)[0] for k in z.files})
+    for n in names:
+        items, offs = oracle.encode_noreorder(z[n + ".A"])
+        assert np.array_equal(offs, z[n + ".offsets"]), n
+        assert np.array_equal(items, z[n + ".items_noreorder"]), n
+    with open(os.path.join(GOLD, "encoder_large.json")) as f:
+        cases = json.load(f)
+    for c in cases:
+        A = spmm.synth_weights(c["M"], c["K"], c["sparsity"], c["row_skewed"], seed=c["seed"])
+        items, offs = oracle.encode_noreorder(A)
+        assert hashlib.sha256(items.tobytes()).hexdigest() == c["items_noreorder_sha256"]
+        assert hashlib.sha256(offs.tobytes()).hexdigest() == c["offsets_sha256"]
+
+
+def test_noreorder_hand_derived(oracle):
+    """Scan order, and pads = the first elements of the scan that are not kept, with their own bits."""
+    A = np.zeros((128, 64), dtype=np.uint16)
+    A[0, 0] = 0x8000   # -0: not kept, becomes the first pad, value bits 0x8000
+    A[0, 1] = 0x7E00   # NaN: not kept, second pad, value bits 0x7e00
+    A[0, 2] = 0x3C00   # 1.0 at (0, 2)
+    A[3, 3] = 0x4000   # 2.0 at (3, 3): swizzled column 3 ^ (3 << 3) = 27
+    items, offs = oracle.encode_noreorder(A)
+    assert list(offs) == [0, 1, 1]
+    assert [int(w) for w in items] == [0x8000 | 0 << 16, 0x7E00 | 1 << 16, 0x3C00 | 2 << 16, 0x4000 | (3 * 64 + 27) << 16]
+
+
+def test_noreorder_same_multiset_as_reordered(oracle, spmm):
+    """Both encoders keep the same elements; only the order inside a tile (and the pad positions) differ."""
+    A = spmm.synth_weights(256, 256, 0.8, True, seed=3)
+    a_items, a_offs = oracle.encode(A)
+    b_items, b_offs = oracle.encode_noreorder(A)
+    assert np.array_equal(a_offs, b_offs)
+    for t in range(len(a_offs) - 2):
+        lo, hi = 4 * a_offs[t], 4 * a_offs[t + 1]
+        x, y = a_items[lo:hi], b_items[lo:hi]
+        assert np.array_equal(np.sort(x[(x & 0xFFFF) != 0]), np.sort(y[(y & 0xFFFF) != 0]))
+    d = oracle.decode(b_items, b_offs, 256, 256)
+    assert np.array_equal(d.astype(np.float32), A.astype(np.float32))
