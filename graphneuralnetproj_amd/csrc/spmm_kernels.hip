@@ -7,37 +7,40 @@
 // (csrc/Reduction_Kernel.cuh:24-47).
 //
 // Design: "load as sparse, compute as dense", one wavefront per work unit.
-//   * A work unit is one 128-row tile row of A times one split-K batch of
-//     64-column tiles, and one wave64 owns it from start to finish: LDS
-//     operations of one wave execute in issue order, which is all the
-//     scatter -> read-back -> clear chain needs, so the loop has no barrier.
-//   * A workgroup is W such waves on consecutive tile rows of the same batch.
-//     They share nothing but the batch's activation slice, staged once into LDS
-//     (one barrier, before the loop), and the fact that W units land on one
-//     compute unit: the host picks W so that the grid is one workgroup per
-//     compute unit where the shape allows it.
-//   * The packed (value,index) words of a tile are streamed from HBM with
-//     non-temporal 128-bit buffer loads into a ring of register slots, a full
-//     tile ahead of their use.  The loads are inline assembly and their
-//     completion is awaited with hand-placed s_waitcnt vmcnt(N): every issue
-//     puts a fixed number of loads in flight, so N is a compile-time constant
-//     and the loads of the next tile stay in flight while this one is consumed.
-//   * A private 16 KiB LDS tile holds the dense 128x64 fp16 image.  It is
-//     cleared once; per tile the wave scatters the values with ds_write_b16 at
-//     byte address 2*index (the index already carries the XOR swizzle that makes
-//     the read-back conflict free), reads the tile back as MFMA operands with
-//     ds_read_b128, issues v_mfma_f32_16x16x32_f16 against activation fragments
-//     read from the staged slice (or, when the slice does not fit, fetched
-//     straight from global memory, where they are L2 resident), and then restores
-//     the zeros by writing 0 to the same addresses.  On gfx950 an LDS write costs
-//     about the same whatever its width, so undoing ~26 scatter instructions is
-//     cheaper than re-clearing 16 KiB.
-//   * TileOffsets of the unit sit in one VGPR (lane i = offset i) and are read
-//     with v_readlane, so the steady-state loop performs no scalar memory reads.
-//   * fp32 accumulators stay in registers over the whole batch; the epilogue
-//     rounds to fp16, transposes through the wave's (by then free) LDS tile and
-//     stores whole 256-byte token rows of one slab of partial sums (or of C
-//     itself when Split_K == 1).
+//   * A work unit is one 128-row tile row of A times a run of 64-column tiles, and one
+//     wave64 owns it from start to finish: LDS operations of one wave execute in issue
+//     order, which is all the scatter -> read-back -> clear chain needs, so the loop has
+//     no barrier.
+//   * A workgroup is W such waves, in one of two layouts the host chooses between:
+//       rows  (KSPLIT = false)  W consecutive tile rows of the same split-K batch; they
+//             can share the batch's activation slice, staged once into LDS (BLDS);
+//       runs  (KSPLIT = true)   the W contiguous runs that one tile row's batch is cut
+//             into; the waves add their accumulators up in LDS at the end, so with
+//             Split_K == 1 the kernel writes C itself.
+//   * The packed (value,index) words of a tile are streamed from HBM with non-temporal
+//     128-bit buffer loads into a ring of two register slots, a full tile ahead of their
+//     use.  The loads are inline assembly and their completion is awaited with hand-placed
+//     s_waitcnt vmcnt(N): every issue puts a fixed number of loads in flight, so N is a
+//     compile-time constant.  A wave keeps one tile in flight: every wave of the chip doing
+//     so already saturates the memory system, and more only lengthens its queues.
+//   * A private 16 KiB LDS tile holds the dense 128x64 fp16 image.  It is cleared once; per
+//     tile the wave scatters the values with ds_write_b16 at byte address 2*index (the index
+//     already carries the XOR swizzle that makes the read-back conflict free), reads the tile
+//     back as MFMA operands with ds_read_b128, issues v_mfma_f32_16x16x32_f16 against the
+//     activation fragments (from the staged slice, or fetched from global memory, where they
+//     are L2 resident), and then restores the zeros by writing 0 to the same addresses.  On
+//     gfx950 an LDS write costs about the same whatever its width, so undoing ~26 scatter
+//     instructions is cheaper than re-clearing 16 KiB.  The words of a tile may come in any
+//     order (the reference's encoder orders them to spread LDS banks; the kernel is memory
+//     bound either way).
+//   * TileOffsets of the unit sit in one VGPR (lane i = offset i) and are read with
+//     v_readlane, so the steady-state loop performs no scalar memory reads.
+//   * fp32 accumulators stay in registers over the whole run; the epilogue rounds to fp16
+//     once.  Split_K > 1 writes slabs of partial sums; in the runs layout the last workgroup
+//     to finish a tile row then adds the slabs up itself (arrival counters in a static device
+//     array, slabs written through and read at system scope), otherwise a second kernel does.
+//   * ROWMAJ takes B as [K][N] and writes [M][N]; strides (ldb, ldo, ldc) and a fused clamp
+//     at zero serve callers that chain layers.
 //
 // Rule for the asynchronous loads: the compiler does not know that the outputs of
 // the load asm statements arrive later.  On every path, each destination register
