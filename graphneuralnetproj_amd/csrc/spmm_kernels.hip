@@ -244,12 +244,12 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
     int kb1 = kb0 + avg;
     kb1 = kb1 < nkb ? kb1 : nkb;
     if (KSPLIT) {
-        // The batch's tiles are dealt to the W waves in contiguous runs.  (Dealing them round
-        // robin, so that the workgroup reads one contiguous stretch at a time, measured slower.)
-        const int run = (kb1 - kb0 + W - 1) / W;
-        kb0 += wave * run;
-        kb0 = kb0 < kb1 ? kb0 : kb1;
-        kb1 = kb0 + run < kb1 ? kb0 + run : kb1;
+        // The batch's tiles are dealt to the W waves in contiguous runs whose lengths differ by at
+        // most one.  (Dealing them round robin, so that the workgroup reads one contiguous stretch
+        // at a time, measured slower.)
+        const int n = kb1 - kb0, q = n / W, r = n - q * W;
+        kb0 += wave * q + (wave < r ? wave : r);
+        kb1 = kb0 + q + (wave < r ? 1 : 0);
     }
     const int ntile = active ? kb1 - kb0 : 0;  // tiles of this wave
     uint8_t* const tile = lds + wave * kTileBytes;
