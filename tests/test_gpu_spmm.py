@@ -568,3 +568,49 @@ def test_product_on_unreordered_encoding(spmm, oracle, N, split_k):
     items, offsets = spmm.InitSparseMatrixA_API_NoReorder(A)
     C, _ = run_gpu(spmm, items, offsets, B, M, N, K, split_k)
     assert_close(C, oracle.gemm_f32(A, B))
+
+
+def test_hip_graph_replays_match_eager(spmm, oracle):
+    """A captured chain (one product with the fused reduction, one without a split, one with the
+    second-kernel reduction) replayed several times, with eager work in between, gives the eager bits."""
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    M, K, N = 1024, 1024, 16
+    A, B, items, offsets = make_case(spmm, M, K, N, 0.8, seed=77)
+    d_items = torch.from_numpy(items.view(np.int32).copy()).to(dev)
+    d_offs = torch.from_numpy(offsets.copy()).to(dev)
+    d_B = torch.from_numpy(np.ascontiguousarray(B).view(np.int16).copy()).to(dev).view(torch.float16)
+    d_x = torch.zeros((N, K), dtype=torch.float16, device=dev)
+    d_y = torch.zeros((N, M), dtype=torch.float16, device=dev)
+    d_z = torch.zeros((N, M), dtype=torch.float16, device=dev)
+    d_u = torch.zeros((N, M), dtype=torch.float16, device=dev)
+    d_W = torch.zeros((4, N, M), dtype=torch.float16, device=dev)
+
+    def chain(stream):
+        # y = A x (Split_K 4, mode 1: fused), z = A y (no split), u = relu(A z) (mode 0: second kernel)
+        spmm.SpMM_SplitK_API_Planned(stream, d_items, d_offs, d_x, d_y, M, N, K, d_W, 4, 1, 4, 0, 0, 0)
+        spmm.SpMM_SplitK_API_Planned(stream, d_items, d_offs, d_y, d_z, M, N, K, None, 1, 1, 8, 0, 0, 0)
+        spmm.SpMM_SplitK_API_Planned(stream, d_items, d_offs, d_z, d_u, M, N, K, d_W, 4, 0, 4, 1, 0,
+                                     spmm.SPMM_FLAG_RELU)
+
+    print("[gpu case] graph capture of three chained products", flush=True)
+    d_x.copy_(d_B)
+    chain(torch.cuda.current_stream())  # eager reference; also arms the kernels' attributes before capture
+    torch.cuda.synchronize()
+    want = d_u.clone()
+    assert torch.isfinite(want).all() and float(want.abs().max()) > 0
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            chain(torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    for rep in range(4):
+        d_y.zero_(); d_z.zero_(); d_u.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(d_u, want), f"replay {rep} differs from the eager result"
+        d_u.zero_()
+        chain(torch.cuda.current_stream())  # eager work between replays
+        torch.cuda.synchronize()
+        assert torch.equal(d_u, want)
