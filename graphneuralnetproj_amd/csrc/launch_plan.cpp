@@ -73,12 +73,6 @@ bool complete_plan(int N, int K, int split_k, bool row_major, LaunchPlan& p)
         return false;
     if (split_k < 1 || p.waves < 1 || p.waves > max_waves(N))
         return false;
-    if (p.mode == 2) {  // one team of N / 16 waves on two shared tile images
-        if (row_major || p.stage_b || (N != 32 && N != 64) || p.waves != N / 16)
-            return false;
-        p.lds_bytes = static_cast<unsigned>(2 * kTileLds);
-        return true;
-    }
     const int nb = column_blocks(N);
     const long nkb = K / kTileCols;
     const long tiles = (nkb - 1) / split_k + 1;  // tiles of the longest batch
@@ -117,26 +111,6 @@ double plan_cost_us(int M, int N, int K, int split_k, const LaunchPlan& p)
     const int W = p.waves;
     const long batch_tiles = (nkb - 1) / split_k + 1;
     long wgs, t;  // workgroups; tiles per wave
-    if (p.mode == 2) {
-        // A team moves one tile stream: for the chip it counts as one wave's worth of traffic per
-        // workgroup, and four (N = 64) or five (N = 32) teams share a compute unit.
-        const long wgs2 = row_tiles * split_k;
-        const long fit2 = N == 64 ? 4 : 5;
-        const double tau_chip2 = (kTileBytes + N * 128.0) / kChipBytesPerUs;
-        double total = kLaunchUs;
-        for (long left = wgs2; left > 0;) {
-            const long n = left < kCUs * fit2 ? left : kCUs * fit2;
-            left -= n;
-            const long per_cu = (n + kCUs - 1) / kCUs;
-            const double chip = static_cast<double>(n) * batch_tiles * tau_chip2;
-            const double lat = kRoundUs + batch_tiles * (kWaveTileUs + 2 * kMfmaTileUs);
-            const double cu = static_cast<double>(per_cu) * batch_tiles * (kTileBytes / kCuBytesPerUs);
-            total += std::pow(std::pow(chip, kNorm) + std::pow(lat, kNorm) + std::pow(cu, kNorm), 1.0 / kNorm);
-        }
-        if (split_k > 1)
-            total += kFusedReduceUs + (2.0 * split_k + 1.0) * M * N * 2.0 / kReduceBytesPerUs;
-        return total;
-    }
     if (p.mode == 0) {
         wgs = (row_tiles + W - 1) / W * split_k;
         t = batch_tiles;
@@ -185,7 +159,7 @@ LaunchPlan plan_launch(int M, int N, int K, int split_k, bool row_major, double*
     }
     LaunchPlan best{0, 1, 0, static_cast<unsigned>(kTileLds)};
     double best_cost = -1.0;
-    for (int mode = 0; mode <= 2; mode++)
+    for (int mode = 0; mode <= 1; mode++)
         for (int w = 1; w <= max_waves(N); w++)
             for (int stage = 0; stage <= (mode == 0 ? 1 : 0); stage++) {
                 LaunchPlan p{mode, w, stage, 0};

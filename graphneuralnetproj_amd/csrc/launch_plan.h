@@ -6,8 +6,7 @@ namespace tcsl {
 // mode 0: the W waves of a workgroup take W consecutive 128-row tile rows of one split-K
 //         batch (stage_b: the batch's activation slice is staged in LDS and shared);
 // mode 1: the W waves of a workgroup split the batch of one tile row among themselves and
-//         add their accumulators up in LDS;
-// mode 2: the W = N / 16 waves of a workgroup (N = 32, 64) share one tile stream, 16 tokens each.
+//         add their accumulators up in LDS.
 struct LaunchPlan {
     int mode;
     int waves;

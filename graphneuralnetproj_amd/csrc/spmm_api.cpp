@@ -135,10 +135,10 @@ int launch_main(void* stream, const void* Compressed_A, const int* TileOffsets, 
 {
     const tcsl::LaunchPlan p = o.forced ? *o.forced : cached_plan(M, N, K, Split_K, o.row_major);
     int page = -1;
-    // Only the layouts whose workgroup owns a single tile row fuse the reduction: their last arriver
+    // Only the layout whose workgroup owns a single tile row fuses the reduction: its last arriver
     // adds up 128 rows.  In the row-sharing layout one workgroup would be left with W x 128 rows of
     // every slab while the rest of the chip idles, which measured slower than the second kernel.
-    if (fused_out && p.mode != 0 && M / tcsl::kTileRows <= 4096)
+    if (fused_out && p.mode == 1 && M / tcsl::kTileRows <= 4096)
         page = counter_page(stream);
     if (fused)
         *fused = page >= 0;

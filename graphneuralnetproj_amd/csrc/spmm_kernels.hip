@@ -687,245 +687,6 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
                          &tcsl_arrivals[fuse_page][blockIdx.x % groups], reinterpret_cast<unsigned int*>(lds));
 }
 
-// N = 32 and 64 as a team: the T = N / 16 waves of a workgroup work on the same tile stream,
-// each owning 16 tokens.  A wave loads and scatters a quarter (half) of a tile's words into a
-// tile image the team shares, all waves read the image back and multiply it with their own
-// tokens, and each restores the zeros under its own words.  Against one wave carrying 64 tokens
-// (128 accumulator registers, 312 VGPRs, one wave per SIMD, nothing overlapping its scatter, MFMA
-// and un-scatter phases) a team wave carries 32 accumulator registers and a quarter of the
-// scatter work, so several teams fit a compute unit and hide each other's phases; the weight
-// stream is still read once.  Two barriers per tile keep the team in step; the image is
-// double buffered so that restoring tile t never meets the scatter of tile t + 1:
-//     scatter(t) | barrier | read + MFMA(t) | barrier | restore(t), scatter(t + 1) into the other image | ...
-// A workgroup is one team on one (128-row tile row, split-K batch) unit; with Split_K > 1 the
-// last team to finish a tile row adds the slabs up (fused_reduction_tail).  Column-major only.
-// Dynamic LDS: 2 x 16 KiB.
-template<int T>
-__global__ __launch_bounds__(T* kWave) void tcsl_spmm_team_kernel(const u32x4* __restrict__ items,
-                                                                  const int* __restrict__ offsets,
-                                                                  const _Float16* __restrict__ B,
-                                                                  _Float16* __restrict__ out, int M, int N, int K,
-                                                                  int split_k, int ldb, int ldo, int relu,
-                                                                  _Float16* __restrict__ fused_out, int ldc,
-                                                                  int fuse_page)
-{
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    constexpr int CH = kVecPerLane / T;  // 64-vector chunks of a segment that this wave loads and scatters
-    constexpr int D = kRing;
-    constexpr int L = 2 + CH;            // loads per issue: two activation fragments, CH word chunks
-    constexpr int kSeg = kVecPerLane * kWave;
-
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const int row_tiles = M / kTileRows;
-    const int rt = blockIdx.x % row_tiles, batch = blockIdx.x / row_tiles;
-    const int nkb = K / kTileCols;
-    const int avg = (nkb - 1) / split_k + 1;  // csrc/SpMM_Kernel.cuh:312-320, clamped to the matrix
-    int kb0 = batch * avg;
-    kb0 = kb0 < nkb ? kb0 : nkb;
-    int kb1 = kb0 + avg;
-    kb1 = kb1 < nkb ? kb1 : nkb;
-    const int ntile = kb1 - kb0;
-    const bool clamp = relu && fuse_page < 0;  // partial sums are never clamped
-
-    const int* toff = offsets + (size_t)rt * nkb + kb0;
-    int wbase = 0;
-    int wreg = toff[lane <= ntile ? lane : ntile];
-
-    // both images start all zero: each wave clears its share
-    {
-        typedef uint64_t __attribute__((may_alias)) u64_a;
-#pragma unroll
-        for (int u = 0; u < 2 * kTileBytes / (T * kWave * 8); u++)
-            *reinterpret_cast<u64_a*>(lds + (u * T + wave) * (kWave * 8) + lane * 8) = 0;
-    }
-    __syncthreads();
-
-    auto tile_range = [&](int i, int& begin, int& end) {
-        if (i + 1 - wbase >= kWave) {
-            wbase = i;
-            const int idx = i + lane;
-            wreg = toff[idx <= ntile ? idx : ntile];
-            settle(wreg);
-        }
-        begin = __builtin_amdgcn_readlane(wreg, i - wbase);
-        end = __builtin_amdgcn_readlane(wreg, i + 1 - wbase);
-    };
-
-    f32x4 acc[8];
-#pragma unroll
-    for (int r = 0; r < 8; r++)
-        acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const int l15 = lane & 15, q = lane >> 4;
-    int a_off[2];
-#pragma unroll
-    for (int s = 0; s < 2; s++)
-        a_off[s] = l15 * 128 + (((s * 4 + q) ^ (lane & 7)) << 4);
-    const _Float16* const bptr = B + (size_t)(wave * 16 + l15) * ldb + (size_t)kb0 * kTileCols + q * 8;
-    // this wave's chunks of a segment: vectors [(wave + T*u) * 64, +64), u < CH
-    int voff[CH];
-#pragma unroll
-    for (int u = 0; u < CH; u++)
-        voff[u] = lane * 16 + (wave + T * u) * 1024;
-    uint32_t vzero = 0, vtwo = 2;
-    asm volatile("" : "+v"(vzero), "+v"(vtwo));
-
-    struct Seg {
-        int tile, begin, n;
-        bool first, last;
-    };
-    struct Cur {
-        int tile, off;
-    };
-    auto make_seg = [&](Cur c, Seg& s, Cur& nxt) {
-        if (c.tile >= ntile) {
-            s = Seg{ntile, 0, 0, true, true};
-            nxt = c;
-            return;
-        }
-        int b, e;
-        tile_range(c.tile, b, e);
-        const int rest = e - b - c.off;
-        s.tile = c.tile;
-        s.begin = b + c.off;
-        s.n = rest < kSeg ? rest : kSeg;
-        s.first = c.off == 0;
-        s.last = rest <= kSeg;
-        nxt = s.last ? Cur{c.tile + 1, 0} : Cur{c.tile, c.off + kSeg};
-    };
-
-    u32x4 regs[D][CH];
-    half8 bfrag[D][2];
-    Seg held[D];
-
-    auto issue = [&](int slot, const Seg& s) {
-        wait_loads<0>();  // one segment in flight per wave, as in the single-wave kernel
-        const bool live = s.tile < ntile;
-        const uint64_t base = reinterpret_cast<uint64_t>(items + s.begin);
-        i32x4 rs = {(int)(uint32_t)base, (int)((uint32_t)(base >> 32) & 0xffff), live ? s.n * 16 : 0, 0x00020000};
-        const int bt = live ? s.tile : ntile - 1;
-#pragma unroll
-        for (int k = 0; k < 2; k++)
-            bfrag[slot][k] = load_activations(bptr + bt * kTileCols + k * 32);
-        static_for<CH>([&](auto uc) {
-            constexpr int u = decltype(uc)::value;
-            regs[slot][u] = load_words<0>(rs, voff[u]);
-        });
-    };
-    auto land = [&](int slot, auto younger) {
-        constexpr int Y = decltype(younger)::value;
-        wait_loads<Y>();
-        static_for<CH>([&](auto uc) { pin(regs[slot][decltype(uc)::value]); });
-#pragma unroll
-        for (int k = 0; k < 2; k++)
-            settle(bfrag[slot][k]);
-    };
-
-    int parity = 0;  // which image the current tile lives in
-    // Every wave of the team sees the same segments, so all take the same path through the barriers.
-    auto consume = [&](int slot, const Seg& s, auto younger) {
-        land(slot, younger);
-        if (s.n == 0)
-            return;  // empty tile or past the end: nothing touched, no barrier
-        uint8_t* const image = lds + parity * kTileBytes;
-        const uint32_t vbase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(image));
-        static_for<CH>([&](auto uc) {
-            constexpr int u = decltype(uc)::value;
-            if (__builtin_expect((wave + T * u) * kWave + lane < s.n, 1))
-                scatter_words<false>(regs[slot][u], vbase, vtwo, vzero);
-        });
-        if (!s.last)
-            return;  // more segments of this tile follow, into the same image
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's scatter writes have landed
-        __syncthreads();                                    // ... and so have everybody's: the image is complete
-#pragma unroll
-        for (int p = 0; p < 2; p++) {
-            half8 afrag[8];
-#pragma unroll
-            for (int r = 0; r < 8; r++)
-                afrag[r] = *reinterpret_cast<const half8*>(image + a_off[p] + r * 2048);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int r = 0; r < 8; r++)
-                acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[r], bfrag[slot][p], acc[r], 0, 0, 0);
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's reads have returned
-        __syncthreads();                                    // ... and everybody's: the image may be changed
-        if (s.first) {
-            static_for<CH>([&](auto uc) {
-                constexpr int u = decltype(uc)::value;
-                if (__builtin_expect((wave + T * u) * kWave + lane < s.n, 1))
-                    scatter_words<true>(regs[slot][u], vbase, vtwo, vzero);
-            });
-        } else {  // earlier segments wrote into the image too and their words are gone: clear this wave's share
-            typedef uint64_t __attribute__((may_alias)) u64_a;
-#pragma unroll
-            for (int u = 0; u < kTileBytes / (T * kWave * 8); u++)
-                *reinterpret_cast<u64_a*>(image + (u * T + wave) * (kWave * 8) + lane * 8) = 0;
-        }
-        parity ^= 1;
-    };
-
-    if (ntile > 0) {
-        Cur ci{0, 0};
-#pragma unroll
-        for (int s = 0; s < D; s++) {
-            Cur nx;
-            make_seg(ci, held[s], nx);
-            ci = nx;
-            issue(s, held[s]);
-        }
-        for (;;) {
-#pragma unroll
-            for (int s = 0; s < D; s++) {
-                consume(s, held[s], std::integral_constant<int, (D - 1) * L>{});
-                Cur nx;
-                make_seg(ci, held[s], nx);
-                ci = nx;
-                issue(s, held[s]);
-            }
-            if (held[0].tile >= ntile)
-                break;
-        }
-#pragma unroll
-        for (int s = 0; s < D; s++)
-            land(s, std::integral_constant<int, 0>{});
-    }
-
-    // Epilogue: acc[r][i] is row r*16 + 4*q + i of token wave*16 + l15.  Through a private
-    // stretch of LDS as [token][128 rows] (token stride 272 B), then 16 bytes per lane.
-    constexpr int kTokStride = 272;
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's last restoring writes
-    __syncthreads();                                      // every wave is done with the images
-    uint8_t* const mine = lds + wave * (16 * kTokStride);
-    _Float16* const oslab = out + (size_t)batch * M * N + (size_t)rt * kTileRows;
-#pragma unroll
-    for (int r = 0; r < 8; r++) {
-        half4 h;
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            h[i] = static_cast<_Float16>(clamp ? fmaxf(acc[r][i], 0.f) : acc[r][i]);
-        *reinterpret_cast<half4*>(mine + l15 * kTokStride + (r * 16 + q * 4) * 2) = h;
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // other lanes read what this lane wrote
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int e = i * kWave + lane;
-        const int tok = e >> 4, part = e & 15;
-        const half8 v = *reinterpret_cast<const half8*>(mine + tok * kTokStride + part * 16);
-        _Float16* dst = oslab + (size_t)(wave * 16 + tok) * ldo + part * 8;
-        if (fuse_page >= 0)
-            store_through(dst, v);
-        else
-            *reinterpret_cast<half8*>(dst) = v;
-    }
-    if (fuse_page < 0)
-        return;
-    __syncthreads();  // the LDS word used next lies inside wave 0's stretch
-    fused_reduction_tail(out, fused_out, M, N, ldc, split_k, relu, rt * kTileRows, kTileRows,
-                         &tcsl_arrivals[fuse_page][rt], reinterpret_cast<unsigned int*>(lds));
-}
-
 // C[n][m] = fp16(sum over slabs of float(W[s][n][m])) (csrc/Reduction_Kernel.cuh:36-46), 8 elements
 // per thread; rows8 = vector length / 8, ldc = elements between two vectors of C (slabs are
 // dense).  The slab loads of a thread are independent; they are issued eight at a time so
@@ -1002,18 +763,6 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
     return static_cast<int>(hipGetLastError());
 }
 
-template<int T>
-int launch_team(hipStream_t stream, const void* items, const int* offsets, const void* B, void* out, int M, int N, int K,
-                int split_k, int ldb, int ldo, int relu, void* fused_out, int ldc, int fuse_page)
-{
-    auto kernel = tcsl_spmm_team_kernel<T>;
-    hipLaunchKernelGGL(kernel, dim3((M / kTileRows) * split_k), dim3(T * kWave), 2 * kTileBytes, stream,
-                       static_cast<const u32x4*>(items), offsets, static_cast<const _Float16*>(B),
-                       static_cast<_Float16*>(out), M, N, K, split_k, ldb, ldo, relu, static_cast<_Float16*>(fused_out), ldc,
-                       fuse_page);
-    return static_cast<int>(hipGetLastError());
-}
-
 }  // namespace
 
 // ---------------------------------------------------------------------------
@@ -1024,8 +773,6 @@ int launch_team(hipStream_t stream, const void* items, const int* offsets, const
 //         stage_b != 0 and N <= 16, share the batch's activation slice in LDS);
 // mode 1: the W waves of a workgroup split the batch of one tile row among themselves and
 //         add their results up in LDS (stage_b must be 0).
-// mode 2: one team of N / 16 waves per workgroup on one (tile row, batch) unit (N = 32, 64;
-//         waves must be N / 16; column-major only).
 // row_major: B is [K][N] and the output [M][N] instead of [N][K] and [N][M] (stage_b must be 0).
 // waves = 1..8 for N <= 32, 1..4 for N = 64; lds_bytes = what the shape needs (the host plans it).
 // ldb, ldo: token strides of B and of the output in elements (column-major; multiples of 8).
@@ -1037,13 +784,6 @@ extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offs
                                 int fuse_page)
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (mode == 2) {  // a team of N / 16 waves per (tile row, batch); column-major, N = 32 or 64
-        if (row_major || stage_b || (N != 32 && N != 64) || waves != N / 16 ||
-            (fuse_page >= 0 && (fuse_page >= kCounterPages || M / kTileRows > kCountersPerPage || split_k < 2 || !fused_out)))
-            return static_cast<int>(hipErrorInvalidValue);
-        return N == 32 ? launch_team<2>(s, items, offsets, B, out, M, N, K, split_k, ldb, ldo, relu, fused_out, ldc, fuse_page)
-                       : launch_team<4>(s, items, offsets, B, out, M, N, K, split_k, ldb, ldo, relu, fused_out, ldc, fuse_page);
-    }
     if (mode != 0 && mode != 1)
         return static_cast<int>(hipErrorInvalidValue);
     if (stage_b && (mode == 1 || row_major || N > 16))

@@ -26,8 +26,6 @@ def candidate_plans(N, tiles_k):
     for S in (1, 2, 3, 4, 6, 8, 12, 16, 24, 32):
         if S <= tiles_k:
             plans += [(S, 1, w, 0) for w in range(3, max_w + 1)]
-    if N >= 32:  # teams of N / 16 waves
-        plans += [(S, 2, N // 16, 0) for S in (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 14, 16, 20, 24, 32) if S <= tiles_k]
     for S in (4, 6, 7, 8, 10, 12, 14, 16, 20, 24, 28, 32):
         if S <= tiles_k:
             if N <= 16:

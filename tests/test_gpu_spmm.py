@@ -284,12 +284,6 @@ PLANS = [
     (1024, 1024, 32, 3, 1, 3, 0),
     (1024, 1024, 64, 1, 1, 4, 0),
     (1024, 1024, 64, 2, 1, 3, 0),
-    (1024, 1024, 32, 1, 2, 2, 0),    # teams: N / 16 waves share one tile stream
-    (1024, 1024, 32, 3, 2, 2, 0),
-    (1024, 1024, 64, 1, 2, 4, 0),
-    (1024, 1024, 64, 4, 2, 4, 0),
-    (128, 64, 64, 1, 2, 4, 0),       # a single tile
-    (256, 64 * 70, 32, 1, 2, 2, 0),  # more than 63 tiles per unit: the offsets window slides
     (256, 64 * 3, 16, 1, 1, 8, 0),   # fewer tiles than waves: five waves have nothing to do
     (256, 64 * 70, 16, 1, 1, 1, 0),  # one wave, more than 63 tiles: the offsets window slides
     (384, 64 * 130, 8, 1, 1, 2, 0),
@@ -541,7 +535,6 @@ def test_fused_reduction_on_two_streams(spmm, oracle):
 
 @pytest.mark.parametrize("N,split_k,mode,waves,stage_b", [
     (32, 8, 0, 1, 0),   # one-wave workgroups, eight resident per compute unit: hundreds finish together
-    (64, 4, 2, 4, 0), (32, 2, 2, 2, 0),   # teams
     (16, 8, 0, 7, 1), (16, 4, 1, 6, 0), (64, 4, 0, 4, 0), (8, 6, 1, 8, 0),
 ])
 def test_fused_reduction_under_load_bit_for_bit(spmm, N, split_k, mode, waves, stage_b):
@@ -621,23 +614,3 @@ def test_hip_graph_replays_match_eager(spmm, oracle):
         chain(torch.cuda.current_stream())  # eager work between replays
         torch.cuda.synchronize()
         assert torch.equal(d_u, want)
-
-
-@pytest.mark.parametrize("N", [32, 64])
-@pytest.mark.parametrize("sparsity", [0.0, 0.4, 0.8, 0.999, 1.0])
-def test_team_kernel_density_sweep(spmm, oracle, N, sparsity):
-    """Teams of N / 16 waves: dense tiles (several segments per tile, whole-image clears), sparse and empty ones."""
-    torch = _torch()
-    dev = torch.device("cuda:0")
-    M, K, split_k = 256, 512, 2
-    A, B, items, offsets = make_case(spmm, M, K, N, sparsity, seed=int(sparsity * 1000) + N)
-    d_items = torch.from_numpy(items.view(np.int32).copy()).to(dev) if len(items) else torch.zeros(4, dtype=torch.int32, device=dev)
-    d_offs = torch.from_numpy(offsets.copy()).to(dev)
-    d_B = torch.from_numpy(np.ascontiguousarray(B).view(np.int16).copy()).to(dev)
-    d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device=dev)
-    d_W = torch.full((split_k, N, M), float("nan"), dtype=torch.float16, device=dev)
-    print(f"[gpu case] team kernel N={N} sparsity={sparsity}", flush=True)
-    spmm.SpMM_SplitK_API_Planned(torch.cuda.current_stream(), d_items, d_offs, d_B, d_C, M, N, K, d_W, split_k, 2,
-                                 N // 16, 0, 0, 0)
-    torch.cuda.synchronize()
-    assert_close(d_C.cpu().numpy(), oracle.gemm_f32(A, B))

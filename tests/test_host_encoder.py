@@ -158,13 +158,10 @@ def test_planner_gives_runnable_plans(spmm):
                 if s > K // 64:
                     continue
                 p = spmm.SpMM_PlanLaunch(M, N, K, s)
-                assert p["mode"] in (0, 1, 2)
+                assert p["mode"] in (0, 1)
                 assert 1 <= p["waves"] <= (8 if N <= 32 else 4)
                 assert p["lds_bytes"] <= 160 * 1024
-                if p["mode"] == 2:  # a team of N / 16 waves on two shared tile images
-                    assert N >= 32 and p["waves"] == N // 16 and p["lds_bytes"] == 32768
-                else:
-                    assert p["lds_bytes"] >= p["waves"] * 16384
+                assert p["lds_bytes"] >= p["waves"] * 16384
                 if p["stage_b"]:
                     assert p["mode"] == 0 and N <= 16
                 assert 0 < p["estimated_us"] < 1e6
@@ -179,7 +176,7 @@ def test_planner_uses_every_compute_unit_on_the_headline_shapes(spmm):
     for (M, K) in [(28672, 7168), (7168, 28672), (36864, 9216), (9216, 36864)]:
         s = spmm.SpMM_SuggestSplitK(M, 16, K)
         p = spmm.SpMM_PlanLaunch(M, 16, K, s)
-        wgs = (M // 128) * s if p["mode"] != 0 else -(-(M // 128) // p["waves"]) * s
+        wgs = (M // 128) * s if p["mode"] == 1 else -(-(M // 128) // p["waves"]) * s
         assert 200 <= wgs <= 512, (M, K, s, p)
 
 
