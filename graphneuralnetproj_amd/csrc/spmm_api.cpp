@@ -13,7 +13,7 @@
 extern "C" {
 int tcsl_launch_spmm(void* stream, const void* items, const int* offsets, const void* B, void* out, int M, int N,
                      int K, int split_k, int mode, int waves, int stage_b, int row_major, unsigned lds_bytes, int ldb,
-                     int ldo, int relu, void* fused_out, int ldc, int fuse_page);
+                     int ldo, int relu, void* fused_out, int ldc, int fuse_page, int dense_waves);
 int tcsl_launch_reduce(void* stream, void* C, const void* W, long rows, long vectors, long ldc, int split_k, int relu);
 int tcsl_launch_copy(void* stream, void* dst, const void* src, long bytes);
 int tcsl_launch_encode_offsets(void* stream, const void* A, int M, int K, int* offsets);
@@ -142,11 +142,22 @@ int launch_main(void* stream, const void* Compressed_A, const int* TileOffsets, 
         page = counter_page(stream);
     if (fused)
         *fused = page >= 0;
-    return tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, out, M, N, K, Split_K, p.mode, p.waves, p.stage_b,
-                            o.row_major ? 1 : 0, p.lds_bytes, ldb, ldo,
+    // The plan's wave count is tuned on 80 % sparse weights.  Sparser ones want every wave the
+    // registers allow (a wave's turnaround per tile becomes the limit), which the host cannot see:
+    // in the K-splitting layout it launches them all and lets each workgroup look at its own tiles.
+    tcsl::LaunchPlan run = p;
+    int dense_waves = 0;
+    if (!o.forced && p.mode == 1 && N <= 32 && p.waves < 8) {
+        tcsl::LaunchPlan all{1, 8, 0, 0};
+        if (tcsl::complete_plan(N, K, Split_K, o.row_major, all)) {
+            run = all;
+            dense_waves = p.waves;
+        }
+    }
+    return tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, out, M, N, K, Split_K, run.mode, run.waves, run.stage_b,
+                            o.row_major ? 1 : 0, run.lds_bytes, ldb, ldo,
                             relu && (Split_K == 1 || page >= 0) ? 1 : 0,  // slabs of partial sums are never clamped
-                            page >= 0 ? fused_out : nullptr,
-                            static_cast<int>(ldc), page);
+                            page >= 0 ? fused_out : nullptr, static_cast<int>(ldc), page, dense_waves);
 }
 
 int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* C, int M, int N,

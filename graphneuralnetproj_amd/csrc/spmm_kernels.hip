@@ -70,6 +70,7 @@ constexpr int kWave = 64;
 constexpr int kVecPerLane = 8;  // 16-byte vectors per lane and ring slot: 512 vectors, i.e. tiles up to 25 % dense in one go
 constexpr int kRing = 2;        // ring slots: one tile being consumed, one in flight
 constexpr unsigned kMaxLdsBytes = 160 * 1024;  // LDS of one gfx950 compute unit
+constexpr int kDenseTileVectors = 300;         // average vectors per tile from which a unit counts as dense (about 85 % sparsity)
 
 // Arrival counters of the fused split-K reduction: one page per caller stream, one counter per
 // group of output rows.  Zero when the module is loaded; the workgroup that brings a counter to
@@ -199,10 +200,11 @@ __device__ __forceinline__ void clear_tile(uint8_t* tile, int lane)
 // of partial sums (through to memory) for rows [row0, row0 + nrows): the last of the Split_K
 // workgroups that share those rows adds the slabs up, in slab order like the separate kernel
 // (csrc/Reduction_Kernel.cuh:36-46), so both paths give the same bits.  `counter` is the rows'
-// arrival count in device memory (zero between calls), `flag` one free LDS word.
+// arrival count in device memory (zero between calls), `flag` one free LDS word, nthreads the
+// number of threads of the workgroup that are still there (the first nthreads).
 __device__ __forceinline__ void fused_reduction_tail(const _Float16* __restrict__ slabs, _Float16* __restrict__ C, int M,
                                                      int N, int ldc, int split_k, int relu, int row0, int nrows,
-                                                     unsigned int* counter, unsigned int* flag)
+                                                     unsigned int* counter, unsigned int* flag, int nthreads)
 {
     // this workgroup's partial sums have reached memory before it is counted
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), on top of what the compiler tracks itself
@@ -215,7 +217,7 @@ __device__ __forceinline__ void fused_reduction_tail(const _Float16* __restrict_
     nrows = nrows < M - row0 ? nrows : M - row0;
     const int per_tok = nrows / 8;
     const size_t slab = (size_t)M * N;
-    for (int c = threadIdx.x; c < per_tok * N; c += blockDim.x) {
+    for (int c = threadIdx.x; c < per_tok * N; c += nthreads) {
         const int tok = c / per_tok, m8 = c - tok * per_tok;
         const _Float16* w0 = slabs + (size_t)tok * M + row0 + m8 * 8;
         float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -266,7 +268,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
                                                                 _Float16* __restrict__ out, int M, int N, int K,
                                                                 int split_k, int ldb, int ldo, int relu,
                                                                 _Float16* __restrict__ fused_out, int ldc,
-                                                                int fuse_page)
+                                                                int fuse_page, int dense_waves)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int VPL = kVecPerLane;
@@ -295,11 +297,24 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
     kb0 = kb0 < nkb ? kb0 : nkb;
     int kb1 = kb0 + avg;
     kb1 = kb1 < nkb ? kb1 : nkb;
+    int Wk = W;  // waves that take part in a K-splitting workgroup
     if (KSPLIT) {
-        // The batch's tiles are dealt to the W waves in contiguous runs whose lengths differ by at
+        const int n = kb1 - kb0;
+        if (dense_waves > 0 && dense_waves < W && n > 0) {
+            // The host launches the waves that sparse tiles want (small tiles: a wave's turnaround
+            // per tile, not the memory system, is the limit, so more waves help) and says how many
+            // dense tiles want; the unit's own density decides.  The others leave before any barrier.
+            const int* u = offsets + (size_t)rt * nkb + kb0;
+            const int vectors = __builtin_amdgcn_readfirstlane(u[n] - u[0]);
+            if (vectors >= kDenseTileVectors * n)
+                Wk = dense_waves;
+            if (wave >= Wk)
+                return;
+        }
+        // The batch's tiles are dealt to the waves in contiguous runs whose lengths differ by at
         // most one.  (Dealing them round robin, so that the workgroup reads one contiguous stretch
         // at a time, measured slower.)
-        const int n = kb1 - kb0, q = n / W, r = n - q * W;
+        const int q = n / Wk, r = n - q * Wk;
         kb0 += wave * q + (wave < r ? wave : r);
         kb1 = kb0 + q + (wave < r ? 1 : 0);
     }
@@ -414,14 +429,16 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
 
     u32x4 regs[D][VPL];
     half8 bfrag[D][BL > 0 ? BL : 1];  // only used when the activations come from global memory
-    Seg held[D];
+    Seg held[D] = {};
 
     // Always exactly L loads, whatever the segment holds, so the wait counts are static.
     auto issue = [&](int slot, const Seg& s) {
-        // Never more than one segment's loads in flight per wave: with the other slot's loads
-        // still outstanding the memory system runs measurably slower (about 4 % on a 165 MB
-        // stream), and they were issued a whole segment ago, so this wait is short.
-        wait_loads<0>();
+        // No more than one full segment's worth (8 KiB) of words in flight per wave: beyond that
+        // the memory system only queues (about 4 % slower on a 165 MB stream at 80 % sparsity,
+        // where two tiles would be 13 KiB).  Two small tiles together (90 % sparsity and up) may
+        // both be in flight, or a wave's 3 KiB at a time would leave it latency bound.
+        if (held[slot ^ 1].n + s.n > kSeg)
+            wait_loads<0>();
         const bool live = s.tile < ntile;
         const uint64_t base = reinterpret_cast<uint64_t>(items + s.begin);
         // descriptor over exactly this segment (nothing at all past the end of the unit)
@@ -589,14 +606,14 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
         for (int r = 0; r < 8; r++)
 #pragma unroll
             for (int c = 0; c < NB; c++)
-                red[((r * W + wave) * NB + c) * kWave + lane] = acc[c][r];
+                red[((r * Wk + wave) * NB + c) * kWave + lane] = acc[c][r];
         __syncthreads();
-        for (int r = wave; r < 8; r += W) {
+        for (int r = wave; r < 8; r += Wk) {
 #pragma unroll
             for (int c = 0; c < NB; c++) {
-                f32x4 sum = red[((r * W) * NB + c) * kWave + lane];
-                for (int w = 1; w < W; w++) {
-                    const f32x4 v = red[((r * W + w) * NB + c) * kWave + lane];
+                f32x4 sum = red[((r * Wk) * NB + c) * kWave + lane];
+                for (int w = 1; w < Wk; w++) {
+                    const f32x4 v = red[((r * Wk + w) * NB + c) * kWave + lane];
 #pragma unroll
                     for (int i = 0; i < 4; i++)
                         sum[i] += v[i];
@@ -684,7 +701,8 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
 
     const int row0 = (KSPLIT ? blockIdx.x % groups : (blockIdx.x % groups) * W) * kTileRows;
     fused_reduction_tail(out, fused_out, M, N, ldc, split_k, relu, row0, (KSPLIT ? 1 : W) * kTileRows,
-                         &tcsl_arrivals[fuse_page][blockIdx.x % groups], reinterpret_cast<unsigned int*>(lds));
+                         &tcsl_arrivals[fuse_page][blockIdx.x % groups], reinterpret_cast<unsigned int*>(lds),
+                         (KSPLIT ? Wk : W) * kWave);
 }
 
 // C[n][m] = fp16(sum over slabs of float(W[s][n][m])) (csrc/Reduction_Kernel.cuh:36-46), 8 elements
@@ -736,7 +754,7 @@ __global__ __launch_bounds__(256) void tcsl_copy_kernel(u32x4* __restrict__ dst,
 template<int NB, bool HALF, bool BLDS, bool KSPLIT, bool ROWMAJ, int MAXW>
 int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const void* B, void* out, int M, int N,
                 int K, int split_k, int waves, unsigned lds_bytes, int ldb, int ldo, int relu, void* fused_out,
-                int ldc, int fuse_page)
+                int ldc, int fuse_page, int dense_waves)
 {
     if (waves < 1 || waves > MAXW || lds_bytes > kMaxLdsBytes)
         return static_cast<int>(hipErrorInvalidValue);
@@ -759,7 +777,7 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
     hipLaunchKernelGGL(kernel, dim3(groups * split_k), dim3(waves * kWave), lds_bytes, stream,
                        static_cast<const u32x4*>(items), offsets, static_cast<const _Float16*>(B),
                        static_cast<_Float16*>(out), M, N, K, split_k, ldb, ldo, relu, static_cast<_Float16*>(fused_out), ldc,
-                       fuse_page);
+                       fuse_page, dense_waves);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -778,10 +796,12 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
 // ldb, ldo: token strides of B and of the output in elements (column-major; multiples of 8).
 // fuse_page >= 0: out = Split_K dense slabs, and the kernel itself reduces them into fused_out
 // (token stride ldc), counting arrivals on that page of counters; at most 4096 row groups.
+// dense_waves (mode 1; 0 = off): of the `waves` launched, only this many work on a unit whose
+// tiles average 300 vectors or more; the kernel looks at each unit's own offsets.
 extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offsets, const void* B, void* out, int M,
                                 int N, int K, int split_k, int mode, int waves, int stage_b, int row_major,
                                 unsigned lds_bytes, int ldb, int ldo, int relu, void* fused_out, int ldc,
-                                int fuse_page)
+                                int fuse_page, int dense_waves)
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (mode != 0 && mode != 1)
@@ -795,7 +815,7 @@ extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offs
     }
 #define TCSL_GO(NB, HALF, BLDS, KS, RM, MAXW) \
     launch_spmm<NB, HALF, BLDS, KS, RM, MAXW>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes, ldb, ldo, relu, \
-                                              fused_out, ldc, fuse_page)
+                                              fused_out, ldc, fuse_page, dense_waves)
 #define TCSL_PICK(NB, HALF, MAXW)                                                                     \
     (row_major ? (mode ? TCSL_GO(NB, HALF, false, true, true, MAXW) : TCSL_GO(NB, HALF, false, false, true, MAXW)) \
                : (mode ? TCSL_GO(NB, HALF, false, true, false, MAXW) : TCSL_GO(NB, HALF, false, false, false, MAXW)))

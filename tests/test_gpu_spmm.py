@@ -614,3 +614,25 @@ def test_hip_graph_replays_match_eager(spmm, oracle):
         chain(torch.cuda.current_stream())  # eager work between replays
         torch.cuda.synchronize()
         assert torch.equal(d_u, want)
+
+
+@pytest.mark.parametrize("N", [16, 32])
+def test_wave_count_follows_each_tile_rows_density(spmm, oracle, N):
+    """A planner shape whose K-splitting plan uses fewer than eight waves: the library launches
+    eight and each workgroup keeps all of them (sparse tile row) or the plan's number (dense one).
+    Rows alternate between 50 % and 97 % sparsity in blocks of 128, so both choices occur in one
+    launch; the planner's own Split_K (> 1) also puts the fused reduction behind both."""
+    M = K = 7168
+    split_k = spmm.SpMM_SuggestSplitK(M, N, K)
+    plan = spmm.SpMM_PlanLaunch(M, N, K, split_k)
+    assert plan["mode"] == 1 and plan["waves"] < 8 and split_k > 1, (plan, split_k)
+    dense = spmm.synth_weights(M, K, 0.5, False, seed=61).view(np.uint16)
+    sparse = spmm.synth_weights(M, K, 0.97, False, seed=62).view(np.uint16)
+    pick = (np.arange(M) // 128) % 2 == 0
+    A = np.where(pick[:, None], dense, sparse).view(np.float16)
+    B = spmm.synth_activations(N, K, seed=63)
+    items, offsets = spmm.InitSparseMatrixA_API(A)
+    per_tile = np.diff(offsets[:-1]).reshape(M // 128, K // 64).mean(axis=1)
+    assert per_tile.min() < 100 and per_tile.max() > 900  # both sides of the kernel's threshold
+    C, _ = run_gpu(spmm, items, offsets, B, M, N, K, split_k)
+    assert_close(C, oracle.gemm_f32(A, B))
