@@ -25,16 +25,22 @@ import numpy as np
 
 
 class Layer:
-    """Device-resident encoded weights of one block: name -> (items, offsets, M, K, split_k)."""
+    """Device-resident weights of one block: name -> (items, offsets, M, K, split_k).
+
+    A matrix that stayed dense on disk (split_k == 0, third_party/ft.patch:1864-1958) is
+    (None, W, M, K, 0) with W the fp16 [K][M] tensor of its file; it goes through the
+    library GEMM, as it goes to cuBLAS in the reference.
+    """
 
     def __init__(self, mats):
         self.mats = mats
 
     def clone(self):
-        return Layer({k: (it.clone(), of, M, K, s) for k, (it, of, M, K, s) in self.mats.items()})
+        return Layer({k: (it.clone() if it is not None else None, of if it is not None else of.clone(), M, K, s)
+                      for k, (it, of, M, K, s) in self.mats.items()})
 
     def bytes(self):
-        return sum(it.numel() * 4 for it, _, _, _, _ in self.mats.values())
+        return sum((it.numel() * 4 if it is not None else of.numel() * 2) for it, of, _, _, _ in self.mats.values())
 
 
 def layer_shapes(h):
@@ -59,31 +65,36 @@ def build_layer(G, torch, dev, h, N, sparsity, seed, keep_dense=False, weight_sc
 class Stack:
     def __init__(self, G, torch, layers, h, N):
         self.G, self.torch, self.layers, self.h, self.N = G, torch, layers, h, N
-        dev = layers[0].mats["qkv"][0].device
+        dev = layers[0].mats["qkv"][1].device
         f16 = torch.float16
         self.x = [torch.zeros((N, h), dtype=f16, device=dev) for _ in range(2)]  # ping-pong layer inputs
         self.qkv = torch.zeros((N, 3 * h), dtype=f16, device=dev)
         self.o = torch.zeros((N, h), dtype=f16, device=dev)
         self.f = torch.zeros((N, 4 * h), dtype=f16, device=dev)
-        max_split = max(s for L in layers for (_, _, _, _, s) in L.mats.values())
+        max_split = max(1, max(s for L in layers for (_, _, _, _, s) in L.mats.values()))
         # one workspace for every product, as the reference's caller keeps (third_party/ft.patch:2762-2765)
         self.ws = torch.zeros((max_split, N, 4 * h), dtype=f16, device=dev)
 
+    def _product(self, stream, mat, src, ldb, dst, ldc, flags=0):
+        it, of, M, K, s = mat
+        if it is not None:
+            self.G.SpMM_SplitK_API_Strided(stream, it, of, src, ldb, dst, ldc, M, self.N, K, self.ws, s, flags)
+        else:  # dense on disk: [N][K] x [K][M] on the library GEMM (torch's current stream)
+            self.torch.mm(src[:, :K], of, out=dst[:, :M])
+            if flags & self.G.SPMM_FLAG_RELU:
+                dst[:, :M].relu_()
+
     def step(self, stream):
         """Enqueue one token step through every layer; returns the buffer holding the result."""
-        G, h, N = self.G, self.h, self.N
+        h = self.h
         cur = 0
         for L in self.layers:
             m = L.mats
             x, nxt = self.x[cur], self.x[cur ^ 1]
-            it, of, M, K, s = m["qkv"]
-            G.SpMM_SplitK_API_Strided(stream, it, of, x, h, self.qkv, 3 * h, M, N, K, self.ws, s, 0)
-            it, of, M, K, s = m["out"]
-            G.SpMM_SplitK_API_Strided(stream, it, of, self.qkv, 3 * h, self.o, h, M, N, K, self.ws, s, 0)
-            it, of, M, K, s = m["ffn1"]
-            G.SpMM_SplitK_API_Strided(stream, it, of, self.o, h, self.f, 4 * h, M, N, K, self.ws, s, G.SPMM_FLAG_RELU)
-            it, of, M, K, s = m["ffn2"]
-            G.SpMM_SplitK_API_Strided(stream, it, of, self.f, 4 * h, nxt, h, M, N, K, self.ws, s, 0)
+            self._product(stream, m["qkv"], x, h, self.qkv, 3 * h)
+            self._product(stream, m["out"], self.qkv, 3 * h, self.o, h)
+            self._product(stream, m["ffn1"], self.o, h, self.f, 4 * h, self.G.SPMM_FLAG_RELU)
+            self._product(stream, m["ffn2"], self.f, 4 * h, nxt, h)
             cur ^= 1
         return self.x[cur]
 
@@ -98,6 +109,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--distinct-weights", action="store_true",
                     help="synthesise and encode every layer separately (default: one layer, copied in HBM)")
+    ap.add_argument("--model-dir", help="run rank 0 of a converted one-rank model directory (<dir>/1-gpu/, written by "
+                                        "graphneuralnetproj_amd.model_files) instead of synthetic weights")
     args = ap.parse_args()
 
     import torch
@@ -108,11 +121,20 @@ def main():
     dev = torch.device("cuda:0")
     h, N = args.hidden, args.tokens
     t0 = time.perf_counter()
-    first, _ = build_layer(G, torch, dev, h, N, args.sparsity, seed=1)
-    layers = [first]
-    for i in range(1, args.layers):
-        layers.append(build_layer(G, torch, dev, h, N, args.sparsity, seed=1 + i)[0] if args.distinct_weights
-                      else first.clone())
+    if args.model_dir:
+        import os
+
+        from . import model_files
+
+        rank_dir = os.path.join(args.model_dir, "1-gpu")
+        args.layers, h = model_files.read_config(rank_dir)
+        layers = model_files.upload_layers(model_files.load_rank(rank_dir, 0, 1), dev, tokens=N)
+    else:
+        first, _ = build_layer(G, torch, dev, h, N, args.sparsity, seed=1)
+        layers = [first]
+        for i in range(1, args.layers):
+            layers.append(build_layer(G, torch, dev, h, N, args.sparsity, seed=1 + i)[0] if args.distinct_weights
+                          else first.clone())
     torch.cuda.synchronize()
     prep_s = time.perf_counter() - t0
     stack = Stack(G, torch, layers, h, N)
@@ -167,13 +189,14 @@ def main():
         "eager_ms": eager_ms, "graph_ms": graph_ms, "graph_matches_eager": graph_matches,
         "config": {"workload": f"{args.layers} layers x (QKV, out-proj, FFN1+ReLU, FFN2), h={h}, N={N}, "
                                f"{args.sparsity * 100:.0f}% sparse",
-                   "weights": "distinct per layer" if args.distinct_weights else "one layer's weights copied per layer"},
+                   "weights": "model directory" if args.model_dir else "distinct per layer" if args.distinct_weights
+                   else "one layer's weights copied per layer"},
         "resident_weight_bytes": weight_bytes,
         "hbm_gbps": weight_bytes / (best_ms * 1e-3) / 1e9,
         "hbm_frac_of_peak": weight_bytes / (best_ms * 1e-3) / 1e9 / 8000.0,
         "effective_tflops": flops / (best_ms * 1e-3) / 1e12,
         "hbm_floor_ms": weight_bytes / 8e12 * 1e3,
-        "prep_s": prep_s, "data": "synthetic",
+        "prep_s": prep_s, "data": "files" if args.model_dir else "synthetic",
     }))
 
 
