@@ -311,12 +311,16 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
             if (wave >= Wk)
                 return;
         }
-        // The batch's tiles are dealt to the waves in contiguous runs whose lengths differ by at
-        // most one.  (Dealing them round robin, so that the workgroup reads one contiguous stretch
-        // at a time, measured slower.)
-        const int q = n / Wk, r = n - q * Wk;
-        kb0 += wave * q + (wave < r ? wave : r);
-        kb1 = kb0 + q + (wave < r ? 1 : 0);
+        // The batch's tiles are dealt to the waves in contiguous runs.  (Dealing them round robin,
+        // so that the workgroup reads one contiguous stretch at a time, measured slower.)  Waves
+        // 4.. share a SIMD with waves 0..3 and issue behind them (the older wave wins the
+        // arbitration; per-wave time stamps show the fifth wave of five about 10 % slower per tile
+        // and the first unaffected), so their runs are 7/8 as long.
+        const int solo = Wk < 4 ? Wk : 4;
+        const int shares = 8 * solo + 7 * (Wk - solo);
+        auto cut = [&](int w) { return (n * (w < 4 ? 8 * w : 32 + 7 * (w - 4)) + shares / 2) / shares; };
+        kb1 = kb0 + cut(wave + 1);
+        kb0 += cut(wave);
     }
     const int ntile = active ? kb1 - kb0 : 0;  // tiles of this wave
     uint8_t* const tile = lds + wave * kTileBytes;
