@@ -108,6 +108,14 @@ __device__ __forceinline__ half8 load_activations(const _Float16* p)
     return r;
 }
 
+// One tile offset per lane, asynchronous like the loads above (to be waited for by hand).
+__device__ __forceinline__ int load_offset(const int* p)
+{
+    int r;
+    asm volatile("global_load_dword %0, %1, off" : "=v"(r) : "v"(p));
+    return r;
+}
+
 // 16 bytes per lane at base + voff (uniform 64-bit base, per-lane 32-bit byte offset)
 __device__ __forceinline__ half8 load_activations_at(const _Float16* base, uint32_t voff)
 {
@@ -254,22 +262,28 @@ __device__ __forceinline__ void fused_reduction_tail(const _Float16* __restrict_
 // fuse_page >= 0 (Split_K > 1, column-major): `out` receives the slabs of partial sums as usual,
 // and the last workgroup to finish a group of rows adds the slabs up into fused_out (token stride
 // ldc, clamped if relu) itself; arrivals are counted in tcsl_arrivals[fuse_page].
-// blockDim.x = W * 64.  Wave w of workgroup g owns tile row (g % groups) * W + w of batch
-// g / groups, groups = ceil(tile rows / W).  NB = number of 16-token column blocks;
+// blockDim.x = W * 64, grid = (groups of tile rows, Split_K).  Wave w of workgroup (g, b) owns
+// tile row g * W + w of batch b; with KSPLIT the workgroup owns tile row g and its waves share
+// the batch.  avg = tiles per batch = ceil((K / 64) / Split_K).  NB = number of 16-token column blocks;
 // ROWMAJ = B is [K][N] and the output [M][N].  HALF = N is 8 (the upper eight columns of the single block are computed on duplicates
 // and dropped); BLDS = the batch's activation slice is staged in LDS; MAXW bounds W and
 // with it the registers a wave may use.
 // Dynamic LDS: W tiles of 16 KiB, then tokens * 128 bytes times tiles_per_batch (BLDS) or times W
 // (ROWMAJ); with KSPLIT at least 8 * W * NB KiB in all (the waves' accumulators meet there).
 template<int NB, bool HALF, bool BLDS, bool KSPLIT, bool ROWMAJ, int MAXW>
-__global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __restrict__ items,
-                                                                const int* __restrict__ offsets,
+__global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __restrict__ offsets,
+                                                                const u32x4* __restrict__ items,
                                                                 const _Float16* __restrict__ B,
-                                                                _Float16* __restrict__ out, int M, int N, int K,
-                                                                int split_k, int ldb, int ldo, int relu,
+                                                                _Float16* __restrict__ out, int K, int avg,
+                                                                int wave_counts, int ldb, int M, int ldo,
                                                                 _Float16* __restrict__ fused_out, int ldc,
-                                                                int fuse_page, int dense_waves)
+                                                                int fuse_page, int relu, int split_k)
 {
+    // (Argument order: the first 14 dwords are preloaded into scalar registers when a wave starts
+    // (-amdgpu-kernarg-preload-count); they are what the way to the first tile's loads needs.
+    // wave_counts = W | dense_waves << 8, W = waves per workgroup = blockDim.x / 64, passed so
+    // that it is among them; the number of tokens is the template's.)
+    const int W = wave_counts & 0xff, dense_waves = wave_counts >> 8;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int VPL = kVecPerLane;
     constexpr int D = kRing;
@@ -284,46 +298,79 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
     static_assert(!(ROWMAJ && BLDS), "row-major activations are not staged");
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // uniform, and known to be
-    const int W = blockDim.x / kWave;
+    // grid: x = group of tile rows (one tile row in the K-splitting layout), y = split-K batch
     const int row_tiles = M / kTileRows;
-    const int groups = KSPLIT ? row_tiles : (row_tiles + W - 1) / W;
-    const int batch = blockIdx.x / groups;
-    const int rt = KSPLIT ? blockIdx.x % groups : (blockIdx.x % groups) * W + wave;
+    const int batch = blockIdx.y;
+    const int rt = KSPLIT ? blockIdx.x : blockIdx.x * W + wave;
     const bool active = rt < row_tiles;
-    // split-K bookkeeping of the reference (csrc/SpMM_Kernel.cuh:312-320), clamped to the matrix
+    // split-K bookkeeping of the reference (csrc/SpMM_Kernel.cuh:312-320), clamped to the matrix;
+    // avg = ceil((K / 64) / split_k), from the host
     const int nkb = K / kTileCols;
-    const int avg = (nkb - 1) / split_k + 1;
     int kb0 = batch * avg;
     kb0 = kb0 < nkb ? kb0 : nkb;
     int kb1 = kb0 + avg;
     kb1 = kb1 < nkb ? kb1 : nkb;
-    int Wk = W;  // waves that take part in a K-splitting workgroup
+    int Wk = W;    // waves that work in a K-splitting workgroup
+    int wreg = 0;  // offsets window: lane l holds the offset of tile wbase + l of this wave's run
+    bool cleared = false;
+    uint8_t* const tile = lds + wave * kTileBytes;
     if (KSPLIT) {
         const int n = kb1 - kb0;
-        if (dense_waves > 0 && dense_waves < W && n > 0) {
-            // The host launches the waves that sparse tiles want (small tiles: a wave's turnaround
-            // per tile, not the memory system, is the limit, so more waves help) and says how many
-            // dense tiles want; the unit's own density decides.  The others leave before any barrier.
-            const int* u = offsets + (size_t)rt * nkb + kb0;
-            const int vectors = __builtin_amdgcn_readfirstlane(u[n] - u[0]);
-            if (vectors >= kDenseTileVectors * n)
-                Wk = dense_waves;
-            if (wave >= Wk)
-                return;
+        const int* u = offsets + (size_t)rt * nkb;  // this tile row's offsets
+        // The batch's tiles are dealt to the working waves in contiguous runs.  (Dealing them
+        // round robin, so that the workgroup reads one contiguous stretch at a time, measured
+        // slower.)  Waves 4.. share a SIMD with waves 0..3 and issue behind them (the older wave
+        // wins the arbitration; per-wave time stamps show the fifth wave of five about 10 %
+        // slower per tile and the first unaffected), so their runs are 7/8 as long: with
+        // share(w) = 8 w for w <= 4, 32 + 7 (w - 4) above, wave w's run starts at tile
+        // round(n share(w) / share(waves)).  The quotient is taken in floating point; x + 1/2 is
+        // never within 1 / (2 * 60) of a multiple of the divisor, far more than the error.
+        auto run = [&](int waves, int& b0, int& b1) {
+            const int shares = waves <= 4 ? 8 * waves : 4 + 7 * waves;
+            const float inv = __builtin_amdgcn_rcpf(static_cast<float>(shares));
+            auto cut = [&](int w) {
+                const int x = n * (w <= 4 ? 8 * w : 4 + 7 * w) + shares / 2;
+                return static_cast<int>((static_cast<float>(x) + 0.5f) * inv);
+            };
+            b0 = kb0 + cut(wave);
+            b1 = kb0 + cut(wave + 1);
+        };
+        int b0, b1;
+        run(W, b0, b1);
+        // The host launches the waves that sparse tiles want (small tiles: a wave's turnaround per
+        // tile, not the memory system, is the limit, so more waves help) and says how many dense
+        // tiles want; the unit's own density decides.  The others stream nothing and wait at the
+        // barrier of the final sum, of which they take their share.  The offsets windows of both
+        // outcomes travel with the two offsets that give the density, so the decision costs no
+        // memory round trip of its own.  (All four loads are issued on every path, adaptive or
+        // not, and waited for in one place: a value that is still on its way must not meet
+        // another at a join, where the compiler would copy it.)
+        const bool adaptive = dense_waves > 0 && dense_waves < W && n > 0;
+        int d0 = kb0, d1 = kb0;
+        if (adaptive && wave < dense_waves)
+            run(dense_waves, d0, d1);
+        int wd = load_offset(u + (d0 + lane <= d1 ? d0 + lane : d1));
+        wreg = load_offset(u + (b0 + lane <= b1 ? b0 + lane : b1));
+        int e0 = load_offset(u + kb0), e1 = load_offset(u + kb1);
+        clear_tile(tile, lane);
+        cleared = true;
+        // (the arguments that are not preloaded are fetched while the offsets are on their way)
+        asm volatile("" ::"s"(relu), "s"(fuse_page), "s"(ldc), "s"(split_k), "s"(fused_out));
+        wait_loads<0>();
+        settle(wd);
+        settle(wreg);
+        settle(e0);
+        settle(e1);
+        if (adaptive && __builtin_amdgcn_readfirstlane(e1 - e0) >= kDenseTileVectors * n) {
+            Wk = dense_waves;
+            b0 = d0;
+            b1 = d1;
+            wreg = wd;
         }
-        // The batch's tiles are dealt to the waves in contiguous runs.  (Dealing them round robin,
-        // so that the workgroup reads one contiguous stretch at a time, measured slower.)  Waves
-        // 4.. share a SIMD with waves 0..3 and issue behind them (the older wave wins the
-        // arbitration; per-wave time stamps show the fifth wave of five about 10 % slower per tile
-        // and the first unaffected), so their runs are 7/8 as long.
-        const int solo = Wk < 4 ? Wk : 4;
-        const int shares = 8 * solo + 7 * (Wk - solo);
-        auto cut = [&](int w) { return (n * (w < 4 ? 8 * w : 32 + 7 * (w - 4)) + shares / 2) / shares; };
-        kb1 = kb0 + cut(wave + 1);
-        kb0 += cut(wave);
+        kb0 = b0;
+        kb1 = b1;
     }
     const int ntile = active ? kb1 - kb0 : 0;  // tiles of this wave
-    uint8_t* const tile = lds + wave * kTileBytes;
     // Activations in LDS, per tile [token][8 granules of 16 B at position g ^ (token & 7)]: the
     // batch's slice, staged once and shared (BLDS), or (ROWMAJ) a one-tile buffer per wave in
     // which the tile's k-major block is turned into token-major MFMA operands.
@@ -333,17 +380,18 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
     // toff[ntile] = end.  Issued first so its latency overlaps the staging below.
     const int* toff = offsets + (size_t)(active ? rt : 0) * nkb + kb0;
     int wbase = 0;
-    int wreg = toff[lane <= ntile ? lane : ntile];
+    if (!KSPLIT)
+        wreg = toff[lane <= ntile ? lane : ntile];
 
     if (BLDS) {
         const int ngran = (kb1 - kb0) * NTOK * 8;  // the whole batch, whatever this wave's own share
-        for (int id = threadIdx.x; id < ngran; id += blockDim.x) {
+        for (int id = threadIdx.x; id < ngran; id += W * kWave) {
             const int j = id / (NTOK * 8), t = (id >> 3) % NTOK, g = id & 7;
             const half8 v = *reinterpret_cast<const half8*>(B + (size_t)t * ldb + (size_t)(kb0 + j) * kTileCols + g * 8);
             *reinterpret_cast<half8*>(bslice + (size_t)j * (NTOK * 128) + t * 128 + ((g ^ (t & 7)) << 4)) = v;
         }
     }
-    if (active)
+    if (active && !cleared)
         clear_tile(tile, lane);
     if (BLDS)
         __syncthreads();  // the only barrier: every wave of the workgroup reaches it
@@ -599,46 +647,63 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
     // global stores are 16 bytes per lane with 16 lanes covering a token's 256 bytes.
     // column-major: C[token][M], this wave's 128 rows start at rt * 128 of every token's vector;
     // row-major: C[M][N], this wave's rows are one contiguous block of 128 * N values
-    _Float16* oslab = out + (size_t)batch * M * N + (size_t)rt * kTileRows * (ROWMAJ ? NTOK : 1);
+    _Float16* oslab = out + (size_t)batch * M * NTOK + (size_t)rt * kTileRows * (ROWMAJ ? NTOK : 1);
     if (KSPLIT) {
-        // Sum the W waves' accumulators through LDS, in wave order.  Layout: [row block r]
-        // [source wave][column block c][lane] x 16 bytes; wave w then owns row blocks w, w + W, ...
+        // Sum the working waves' accumulators through LDS, in wave order.  Each parks its own in
+        // its own tile, [row block r][column block c][lane] x 16 bytes (two tiles' worth at
+        // N = 64, which then takes a barrier before as well); every launched wave w, working or
+        // not, then owns the (r, c) cells w, w + W, ...  The sum is specialised by the number of
+        // working waves: a vector instruction takes four cycles, so selects or a loop would cost
+        // more than the additions themselves.
+        constexpr int kCells = 8 * NB;
+        constexpr bool kOwnTile = kCells * kWave * 16 <= kTileBytes;
         f32x4* const red = reinterpret_cast<f32x4*>(lds);
+        const int wave_stride = kOwnTile ? kTileBytes / 16 : kCells * kWave;  // in f32x4
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's last clearing writes
-        __syncthreads();                                      // every wave is done with its tile
+        if (!kOwnTile)
+            __syncthreads();                                  // every wave is done with its tile
+        if (wave < Wk) {
 #pragma unroll
-        for (int r = 0; r < 8; r++)
+            for (int r = 0; r < 8; r++)
 #pragma unroll
-            for (int c = 0; c < NB; c++)
-                red[((r * Wk + wave) * NB + c) * kWave + lane] = acc[c][r];
+                for (int c = 0; c < NB; c++)
+                    red[wave * wave_stride + (r * NB + c) * kWave + lane] = acc[c][r];
+        }
         __syncthreads();
-        for (int r = wave; r < 8; r += Wk) {
+        for (int cell = wave; cell < kCells; cell += W) {
+            const int r = cell / NB, c = cell % NB;
+            const f32x4* const src = red + cell * kWave + lane;
+            f32x4 sum = src[0];
+            static_for<MAXW - 1>([&](auto wc) {
+                constexpr int WK = decltype(wc)::value + 2;  // 2 .. MAXW working waves
+                if (Wk == WK) {
+                    f32x4 part[WK];
 #pragma unroll
-            for (int c = 0; c < NB; c++) {
-                f32x4 sum = red[((r * Wk) * NB + c) * kWave + lane];
-                for (int w = 1; w < Wk; w++) {
-                    const f32x4 v = red[((r * Wk + w) * NB + c) * kWave + lane];
+                    for (int w = 1; w < WK; w++)
+                        part[w] = src[w * wave_stride];
 #pragma unroll
-                    for (int i = 0; i < 4; i++)
-                        sum[i] += v[i];
+                    for (int w = 1; w < WK; w++)
+#pragma unroll
+                        for (int i = 0; i < 4; i++)
+                            sum[i] += part[w][i];
                 }
-                half4 h;
+            });
+            half4 h;
 #pragma unroll
-                for (int i = 0; i < 4; i++)
-                    h[i] = static_cast<_Float16>(clamp ? fmaxf(sum[i], 0.f) : sum[i]);
-                // rows r*16 + 4*q .. +3 of token c*16 + l15
-                if (!(HALF && l15 >= 8)) {
-                    if (ROWMAJ) {
+            for (int i = 0; i < 4; i++)
+                h[i] = static_cast<_Float16>(clamp ? fmaxf(sum[i], 0.f) : sum[i]);
+            // rows r*16 + 4*q .. +3 of token c*16 + l15
+            if (!(HALF && l15 >= 8)) {
+                if (ROWMAJ) {
 #pragma unroll
-                        for (int i = 0; i < 4; i++)  // the 16 tokens of a row are adjacent
-                            oslab[(r * 16 + q * 4 + i) * NTOK + c * 16 + l15] = h[i];
-                    } else {  // the four q-lanes of a token cover 32 bytes
-                        _Float16* dst = oslab + (size_t)(c * 16 + l15) * ldo + r * 16 + q * 4;
-                        if (fuse_page >= 0)
-                            store_through(dst, h);
-                        else
-                            *reinterpret_cast<half4*>(dst) = h;
-                    }
+                    for (int i = 0; i < 4; i++)  // the 16 tokens of a row are adjacent
+                        oslab[(r * 16 + q * 4 + i) * NTOK + c * 16 + l15] = h[i];
+                } else {  // the four q-lanes of a token cover 32 bytes
+                    _Float16* dst = oslab + (size_t)(c * 16 + l15) * ldo + r * 16 + q * 4;
+                    if (fuse_page >= 0)
+                        store_through(dst, h);
+                    else
+                        *reinterpret_cast<half4*>(dst) = h;
                 }
             }
         }
@@ -703,10 +768,10 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const u32x4* __r
     if (ROWMAJ || fuse_page < 0)
         return;
 
-    const int row0 = (KSPLIT ? blockIdx.x % groups : (blockIdx.x % groups) * W) * kTileRows;
-    fused_reduction_tail(out, fused_out, M, N, ldc, split_k, relu, row0, (KSPLIT ? 1 : W) * kTileRows,
-                         &tcsl_arrivals[fuse_page][blockIdx.x % groups], reinterpret_cast<unsigned int*>(lds),
-                         (KSPLIT ? Wk : W) * kWave);
+    const int row0 = (KSPLIT ? blockIdx.x : blockIdx.x * W) * kTileRows;
+    fused_reduction_tail(out, fused_out, M, NTOK, ldc, split_k, relu, row0, (KSPLIT ? 1 : W) * kTileRows,
+                         &tcsl_arrivals[fuse_page][blockIdx.x], reinterpret_cast<unsigned int*>(lds),
+                         W * kWave);
 }
 
 // C[n][m] = fp16(sum over slabs of float(W[s][n][m])) (csrc/Reduction_Kernel.cuh:36-46), 8 elements
@@ -778,10 +843,13 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
     }
     const int row_tiles = M / kTileRows;
     const int groups = KSPLIT ? row_tiles : (row_tiles + waves - 1) / waves;
-    hipLaunchKernelGGL(kernel, dim3(groups * split_k), dim3(waves * kWave), lds_bytes, stream,
-                       static_cast<const u32x4*>(items), offsets, static_cast<const _Float16*>(B),
-                       static_cast<_Float16*>(out), M, N, K, split_k, ldb, ldo, relu, static_cast<_Float16*>(fused_out), ldc,
-                       fuse_page, dense_waves);
+    const int nkb = K / kTileCols;
+    if (split_k > 65535)
+        return static_cast<int>(hipErrorInvalidValue);
+    hipLaunchKernelGGL(kernel, dim3(groups, split_k), dim3(waves * kWave), lds_bytes, stream,
+                       offsets, static_cast<const u32x4*>(items), static_cast<const _Float16*>(B),
+                       static_cast<_Float16*>(out), K, (nkb - 1) / split_k + 1, waves | dense_waves << 8, ldb, M, ldo,
+                       static_cast<_Float16*>(fused_out), ldc, fuse_page, relu, split_k);
     return static_cast<int>(hipGetLastError());
 }
 
