@@ -126,6 +126,7 @@ struct CallOptions {
     void* ev_begin = nullptr; // events recorded around the main kernel
     void* ev_end = nullptr;
     const tcsl::LaunchPlan* forced = nullptr;
+    bool adaptive_waves = false;  // with `forced`: launch it the way a planned call would be
 };
 
 // fused_out != nullptr asks for the fused reduction; *fused says whether it was possible.
@@ -147,7 +148,7 @@ int launch_main(void* stream, const void* Compressed_A, const int* TileOffsets, 
     // in the K-splitting layout it launches them all and lets each workgroup look at its own tiles.
     tcsl::LaunchPlan run = p;
     int dense_waves = 0;
-    if (!o.forced && p.mode == 1 && N <= 32 && p.waves < 8) {
+    if ((!o.forced || o.adaptive_waves) && p.mode == 1 && N <= 32 && p.waves < 8) {
         tcsl::LaunchPlan all{1, 8, 0, 0};
         if (tcsl::complete_plan(N, K, Split_K, o.row_major, all)) {
             run = all;
@@ -202,11 +203,13 @@ extern "C" int SpMM_SplitK_API_Planned(void* stream, const void* Compressed_A, c
 {
     tcsl::LaunchPlan p{Mode, Waves, StageB, 0};
     if (!tcsl::complete_plan(N, K > 0 ? K : 64, Split_K, RowMajor != 0, p) ||
-        (Flags & ~(SPMM_FLAG_RELU | SPMM_FLAG_SEPARATE_REDUCTION)) != 0 || (RowMajor && (Flags & SPMM_FLAG_RELU)))
+        (Flags & ~(SPMM_FLAG_RELU | SPMM_FLAG_SEPARATE_REDUCTION | SPMM_FLAG_ADAPTIVE_WAVES)) != 0 ||
+        (RowMajor && (Flags & SPMM_FLAG_RELU)))
         return tcsl_error_invalid_value();
     CallOptions o;
     o.relu = (Flags & SPMM_FLAG_RELU) != 0;
     o.separate_reduction = (Flags & SPMM_FLAG_SEPARATE_REDUCTION) != 0;
+    o.adaptive_waves = (Flags & SPMM_FLAG_ADAPTIVE_WAVES) != 0;
     o.row_major = RowMajor != 0;
     o.forced = &p;
     return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, o);

@@ -229,6 +229,7 @@ def SpMM_SplitK_API_RowMajor(stream, A, Compressed_A, TileOffsets, B, C, M_Globa
 
 SPMM_FLAG_RELU = 1
 SPMM_FLAG_SEPARATE_REDUCTION = 2
+SPMM_FLAG_ADAPTIVE_WAVES = 4  # SpMM_SplitK_API_Planned only
 
 
 def SpMM_SplitK_API_Strided(stream, Compressed_A, TileOffsets, B, ldb, C, ldc, M_Global, N_Global, K_Global,

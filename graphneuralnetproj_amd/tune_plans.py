@@ -73,7 +73,8 @@ def main():
             def call(i, plan):
                 S, mode, w, st = plan
                 return lib.SpMM_SplitK_API_Planned(stream, d_items[i % copies].data_ptr(), d_offs.data_ptr(),
-                                                   d_B.data_ptr(), d_C.data_ptr(), M, N, K, d_W.data_ptr(), S, mode, w, st, 0, 0)
+                                                   d_B.data_ptr(), d_C.data_ptr(), M, N, K, d_W.data_ptr(), S, mode, w, st, 0,
+                                                   G.SPMM_FLAG_ADAPTIVE_WAVES)  # as a planned call launches it
 
             S0 = G.SpMM_SuggestSplitK(M, N, K)
             G.SpMM_SplitK_API(None, None, d_items[0], d_offs, d_B, d_C, M, N, K, d_W, S0)

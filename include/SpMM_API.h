@@ -118,6 +118,8 @@ SPMM_EXPORT int SpMM_SplitK_API_RowMajor(void* stream, const void* A, const void
  */
 #define SPMM_FLAG_RELU 1
 #define SPMM_FLAG_SEPARATE_REDUCTION 2 /* Split_K > 1: always run the reduction as its own kernel */
+#define SPMM_FLAG_ADAPTIVE_WAVES 4     /* SpMM_SplitK_API_Planned only: treat Waves (Mode 1, N <= 32) the way a planned
+                                          call does, as the count for dense tile rows, and launch eight */
 SPMM_EXPORT int SpMM_SplitK_API_Strided(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
                                         long ldb, void* C, long ldc, int M_Global, int N_Global, int K_Global,
                                         void* Reduction_Workspace, int Split_K, int Flags);
