@@ -324,13 +324,15 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         // slower per tile and the first unaffected), so their runs are 7/8 as long: with
         // share(w) = 8 w for w <= 4, 32 + 7 (w - 4) above, wave w's run starts at tile
         // round(n share(w) / share(waves)).  The quotient is taken in floating point; x + 1/2 is
-        // never within 1 / (2 * 60) of a multiple of the divisor, far more than the error.
+        // never within 1 / (2 * 60) of a multiple of the divisor, far more than the error (and
+        // beyond 2^24 / 60 tiles per batch, where it is not, neighbours still compute the same cuts).
         auto run = [&](int waves, int& b0, int& b1) {
             const int shares = waves <= 4 ? 8 * waves : 4 + 7 * waves;
             const float inv = __builtin_amdgcn_rcpf(static_cast<float>(shares));
-            auto cut = [&](int w) {
+            auto cut = [&](int w) {  // cut(0) = 0, cut(waves) = n whatever the rounding does
                 const int x = n * (w <= 4 ? 8 * w : 4 + 7 * w) + shares / 2;
-                return static_cast<int>((static_cast<float>(x) + 0.5f) * inv);
+                const int c = static_cast<int>((static_cast<float>(x) + 0.5f) * inv);
+                return w >= waves ? n : (c < n ? c : n);
             };
             b0 = kb0 + cut(wave);
             b1 = kb0 + cut(wave + 1);

@@ -636,3 +636,32 @@ def test_wave_count_follows_each_tile_rows_density(spmm, oracle, N):
     assert per_tile.min() < 100 and per_tile.max() > 900  # both sides of the kernel's threshold
     C, _ = run_gpu(spmm, items, offsets, B, M, N, K, split_k)
     assert_close(C, oracle.gemm_f32(A, B))
+
+
+@pytest.mark.parametrize("flags", [0, 4])
+def test_every_partition_of_a_tile_row_among_the_waves(spmm, oracle, flags):
+    """The K-splitting layout deals a batch's tiles to 1..8 waves in runs of unequal length.  One
+    tile row, 1..113 tiles, every wave count, with exactly representable data (A in {0, 1},
+    B in {-5..3}: the reference's own near-exact test values, kernel_benchmark/spmm_test_utils.h:111-141),
+    so a tile left out or taken twice changes the result by whole numbers.  flags = 4 launches
+    eight waves and lets the kernel choose, as a planned call does."""
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    M, N = 128, 16
+    rng = np.random.default_rng(17)
+    for tiles in (1, 2, 3, 4, 5, 7, 8, 9, 13, 23, 31, 61, 64, 65, 100, 113):
+        K = 64 * tiles
+        A = (rng.random((M, K)) < 0.2).astype(np.float16)
+        B = rng.integers(-5, 4, size=(N, K)).astype(np.float16)
+        ref = oracle.gemm_f32(A, B)
+        items, offsets = spmm.InitSparseMatrixA_API(A)
+        d_items = torch.from_numpy(items.view(np.int32).copy()).to(dev)
+        d_offs = torch.from_numpy(offsets.copy()).to(dev)
+        d_B = torch.from_numpy(B.view(np.int16).copy()).to(dev)
+        for waves in range(1, 9):
+            d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device=dev)
+            print(f"[gpu case] partition tiles={tiles} waves={waves} flags={flags}", flush=True)
+            spmm.SpMM_SplitK_API_Planned(torch.cuda.current_stream(), d_items, d_offs, d_B, d_C, M, N, K, None, 1, 1,
+                                         waves, 0, 0, flags)
+            torch.cuda.synchronize()
+            assert np.array_equal(d_C.cpu().numpy(), ref.astype(np.float16)), (tiles, waves)  # integers: exact
