@@ -28,12 +28,12 @@ constexpr double kChipBytesPerUs = 7.0e6;   // whole-chip stream rate
 constexpr double kCuBytesPerUs = 39.2e3;    // what one compute unit can pull on its own
 constexpr double kWaveTileUs = 0.367;       // a lone wave's turnaround per tile (latency bound)
 constexpr double kMfmaTileUs = 0.199;       // serial MFMA + LDS time per tile and 16-token block
-constexpr double kRoundUs = 4.74;           // start-up and drain of one round of workgroups
+constexpr double kRoundUs = 4.00;           // start-up and drain of one round of workgroups
 constexpr double kNorm = 3.30;              // exponent that blends the three bounds
 constexpr double kCrowdPenalty = 0.043;     // per resident wave above kCrowdWaves on a unit
 constexpr double kCrowdWaves = 6.64;
 constexpr double kGlobalBPenalty = 0.30;   // mode 0, N <= 16, slice not staged
-constexpr double kModeKPenalty = 0.086;     // mode 1: activations from L2, reduction in LDS
+constexpr double kModeKPenalty = 0.020;     // mode 1: activations from L2, reduction in LDS
 constexpr double kReduceUs = 3.44;          // fixed cost of the reduction as a second kernel (mode 0)
 constexpr double kFusedReduceUs = 2.19;     // ... and inside the main kernel (mode 1)
 constexpr double kReduceBytesPerUs = 4.50e6;

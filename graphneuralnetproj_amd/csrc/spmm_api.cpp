@@ -253,7 +253,7 @@ extern "C" int SpMM_SplitK_Partials(void* stream, const void* Compressed_A, cons
     if (N != 8 && N != 16 && N != 32 && N != 64)
         return tcsl_error_unknown();
     if (M <= 0 || K <= 0 || M % tcsl::kTileRows != 0 || K % tcsl::kTileCols != 0 || Split_K < 1 ||
-        static_cast<long>(M / tcsl::kTileRows) * Split_K > 0x7fffffffL)
+        Split_K > 65535)
         return tcsl_error_invalid_value();
     if (!Compressed_A || !TileOffsets || !B || !Partials)
         return tcsl_error_invalid_value();
@@ -299,8 +299,8 @@ int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, 
         std::fprintf(stderr, "SpMM_SplitK_API: null device pointer\n");
         return tcsl_error_invalid_value();
     }
-    // the launch grid is at most (M/128) * Split_K workgroups
-    if (static_cast<long>(M / tcsl::kTileRows) * Split_K > 0x7fffffffL) {
+    // the launch grid is (groups of tile rows) x Split_K workgroups, and a grid's second dimension ends at 65535
+    if (Split_K > 65535) {
         std::fprintf(stderr, "SpMM_SplitK_API: Split_K=%d too large for M=%d\n", Split_K, M);
         return tcsl_error_invalid_value();
     }

@@ -84,7 +84,7 @@ SPMM_EXPORT int InitSparseMatrixA_API_NoReorder(const uint16_t* A_h, int M, int 
  * Accumulation is fp32.  Returns the hipError_t value: 0 on success;
  * hipErrorUnknown, after printing the reference's message, for N outside
  * {8, 16, 32, 64} (csrc/SpMM_API.cu:192-193); hipErrorInvalidValue for M % 128,
- * K % 64, Split_K < 1 or a null pointer (the reference checks these only in
+ * K % 64, Split_K < 1, Split_K > 65535 or a null pointer (the reference checks these only in
  * debug builds, :93-98, and requires M % 256).  Nothing is launched on error.
  * Thread safe.  The in-launch reduction counts arrivals in a small static device array, one
  * page per stream handle (64 pages; further streams fall back to the second kernel): calls on

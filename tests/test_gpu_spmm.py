@@ -255,6 +255,8 @@ def test_errors_launch_nothing(spmm):
         spmm.SpMM_SplitK_API(None, None, t, t, t, C, 128, 16, 64, t, 0)   # Split_K
     with pytest.raises(spmm.SpMMError):
         spmm.SpMM_SplitK_API(None, None, t, t, t, C, 128, 16, 64, None, 2)  # no workspace
+    with pytest.raises(spmm.SpMMError):
+        spmm.SpMM_SplitK_API(None, None, t, t, t, C, 128, 16, 64, t, 65536)  # beyond the launch grid
     torch.cuda.synchronize()
     assert (C == 5.0).all()
 
