@@ -17,7 +17,8 @@ import time
 
 import numpy as np
 
-OPT_SHAPES = "28672x7168,7168x28672,21504x7168,7168x7168,27648x9216,9216x9216,36864x9216,9216x36864"
+OPT_SHAPES = ("28672x7168,7168x28672,21504x7168,7168x7168,27648x9216,9216x9216,36864x9216,9216x36864,"
+              "36864x12288,12288x12288,49152x12288,12288x49152")  # OPT-30B, 66B and 175B on one GPU
 
 
 def candidate_plans(N, tiles_k):
