@@ -28,9 +28,11 @@
 //     already carries the XOR swizzle that makes the read-back conflict free), reads the tile
 //     back as MFMA operands with ds_read_b128, issues v_mfma_f32_16x16x32_f16 against the
 //     activation fragments (from the staged slice, or fetched from global memory, where they
-//     are L2 resident), and then restores the zeros by writing 0 to the same addresses.  On
-//     gfx950 an LDS write costs about the same whatever its width, so undoing ~26 scatter
-//     instructions is cheaper than re-clearing 16 KiB.  The words of a tile may come in any
+//     are L2 resident), and then restores the zeros by writing 0 to the same addresses (kept
+//     in registers where there is room: a wave is busy about 1 us per tile, which five waves
+//     per compute unit only just turn into more than the memory delivers, so every vector
+//     instruction saved shows).  Undoing ~26 scatter instructions is cheaper than re-clearing
+//     16 KiB, which costs as much LDS bandwidth as reading the tile.  The words of a tile may come in any
 //     order (the reference's encoder orders them to spread LDS banks; the kernel is memory
 //     bound either way).
 //   * TileOffsets of the unit sit in one VGPR (lane i = offset i) and are read with
@@ -193,6 +195,22 @@ __device__ __forceinline__ void scatter_words(u32x4 w, uint32_t base, uint32_t t
                      : "=&v"(a0), "=&v"(a1), "=&v"(a2), "=&v"(a3)
                      : "v"(w.x), "v"(w.y), "v"(w.z), "v"(w.w), "v"(base), "v"(two), "v"(zero)
                      : "memory");
+}
+// The same, keeping the four addresses (and, below, writing zero to kept addresses).
+__device__ __forceinline__ void scatter_words_keep(u32x4 w, uint32_t base, uint32_t two, uint32_t (&a)[4])
+{
+    asm volatile(TCSL_ADDR("%0", "%4") TCSL_ADDR("%1", "%5") TCSL_ADDR("%2", "%6") TCSL_ADDR("%3", "%7")
+                 "ds_write_b16 %0, %4\n ds_write_b16 %1, %5\n ds_write_b16 %2, %6\n ds_write_b16 %3, %7\n"
+                 : "=&v"(a[0]), "=&v"(a[1]), "=&v"(a[2]), "=&v"(a[3])
+                 : "v"(w.x), "v"(w.y), "v"(w.z), "v"(w.w), "v"(base), "v"(two)
+                 : "memory");
+}
+__device__ __forceinline__ void clear_words(const uint32_t (&a)[4], uint32_t zero)
+{
+    asm volatile("ds_write_b16 %0, %4\n ds_write_b16 %1, %4\n ds_write_b16 %2, %4\n ds_write_b16 %3, %4\n"
+                 :
+                 : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(zero)
+                 : "memory");
 }
 #undef TCSL_ADDR
 
@@ -545,10 +563,16 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         land(slot, younger);
         if (s.n == 0)
             return;  // empty tile or past the end
+        constexpr bool kKeep = NB == 1;  // room for the 32 addresses only with one column block
+        uint32_t kept[kKeep ? VPL : 1][4];
         static_for<VPL>([&](auto uc) {
             constexpr int u = decltype(uc)::value;
-            if (__builtin_expect(u * kWave + lane < s.n, 1))  // lanes past the segment's end sit out
-                scatter_words<false>(regs[slot][u], vbase, vtwo, vzero);
+            if (__builtin_expect(u * kWave + lane < s.n, 1)) {  // lanes past the segment's end sit out
+                if constexpr (kKeep)
+                    scatter_words_keep(regs[slot][u], vbase, vtwo, kept[u]);
+                else
+                    scatter_words<false>(regs[slot][u], vbase, vtwo, vzero);
+            }
         });
         if (!s.last)
             return;  // more segments of this tile follow
@@ -608,8 +632,12 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         } else {
             static_for<VPL>([&](auto uc) {
                 constexpr int u = decltype(uc)::value;
-                if (__builtin_expect(u * kWave + lane < s.n, 1))
-                    scatter_words<true>(regs[slot][u], vbase, vtwo, vzero);
+                if (__builtin_expect(u * kWave + lane < s.n, 1)) {
+                    if constexpr (kKeep)
+                        clear_words(kept[u], vzero);
+                    else
+                        scatter_words<true>(regs[slot][u], vbase, vtwo, vzero);
+                }
             });
         }
     };
