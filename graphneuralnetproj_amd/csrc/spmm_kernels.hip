@@ -565,14 +565,39 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
             return;  // empty tile or past the end
         constexpr bool kKeep = NB == 1;  // room for the 32 addresses only with one column block
         uint32_t kept[kKeep ? VPL : 1][4];
-        static_for<VPL>([&](auto uc) {
-            constexpr int u = decltype(uc)::value;
-            if (__builtin_expect(u * kWave + lane < s.n, 1)) {  // lanes past the segment's end sit out
-                if constexpr (kKeep)
-                    scatter_words_keep(regs[slot][u], vbase, vtwo, kept[u]);
-                else
-                    scatter_words<false>(regs[slot][u], vbase, vtwo, vzero);
+        // One code path per number of full 64-vector chunks (a uniform switch): those run
+        // unguarded, the one partial chunk under a lane mask, the rest not at all.  (A lane mask
+        // per chunk costs a compare and three scalar instructions each, twice per tile.)
+        const int full = s.n >> 6;
+        const bool in_part = (full << 6) + lane < s.n;  // this lane's vector of the partial chunk exists
+        auto by_chunks = [&](auto&& op) {
+            auto run = [&](auto pc) {
+                constexpr int P = decltype(pc)::value;
+                static_for<P>([&](auto uc) { op(uc); });
+                if constexpr (P < VPL) {
+                    if (in_part)
+                        op(pc);
+                }
+            };
+            switch (full) {
+                case 0: run(std::integral_constant<int, 0>{}); break;
+                case 1: run(std::integral_constant<int, 1>{}); break;
+                case 2: run(std::integral_constant<int, 2>{}); break;
+                case 3: run(std::integral_constant<int, 3>{}); break;
+                case 4: run(std::integral_constant<int, 4>{}); break;
+                case 5: run(std::integral_constant<int, 5>{}); break;
+                case 6: run(std::integral_constant<int, 6>{}); break;
+                case 7: run(std::integral_constant<int, 7>{}); break;
+                default: run(std::integral_constant<int, 8>{}); break;
             }
+        };
+        static_assert(VPL == 8, "the switch above lists 0..8 full chunks");
+        by_chunks([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            if constexpr (kKeep)
+                scatter_words_keep(regs[slot][u], vbase, vtwo, kept[u]);
+            else
+                scatter_words<false>(regs[slot][u], vbase, vtwo, vzero);
         });
         if (!s.last)
             return;  // more segments of this tile follow
@@ -630,14 +655,12 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         if (!s.first) {
             clear_tile(tile, lane);
         } else {
-            static_for<VPL>([&](auto uc) {
+            by_chunks([&](auto uc) {
                 constexpr int u = decltype(uc)::value;
-                if (__builtin_expect(u * kWave + lane < s.n, 1)) {
-                    if constexpr (kKeep)
-                        clear_words(kept[u], vzero);
-                    else
-                        scatter_words<true>(regs[slot][u], vbase, vtwo, vzero);
-                }
+                if constexpr (kKeep)
+                    clear_words(kept[u], vzero);
+                else
+                    scatter_words<true>(regs[slot][u], vbase, vtwo, vzero);
             });
         }
     };
