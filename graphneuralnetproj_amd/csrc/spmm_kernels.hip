@@ -69,7 +69,9 @@ constexpr int kTileRows = 128;  // rows of one encoded tile
 constexpr int kTileCols = 64;   // columns of one encoded tile
 constexpr int kTileBytes = kTileRows * kTileCols * 2;
 constexpr int kWave = 64;
-constexpr int kVecPerLane = 8;  // 16-byte vectors per lane and ring slot: 512 vectors, i.e. tiles up to 25 % dense in one go
+constexpr int kVecPerLane = 8;       // 16-byte vectors per lane and ring slot: 512 vectors, i.e. tiles up to 25 % dense in one go
+constexpr int kVecPerLaneLong = 10;  // ... and for units whose tiles mostly exceed that: 640 vectors, 31 % dense
+constexpr int kLongTileVectors = 498;  // average vectors per tile from which a unit takes the long segments
 constexpr int kRing = 2;        // ring slots: one tile being consumed, one in flight
 constexpr unsigned kMaxLdsBytes = 160 * 1024;  // LDS of one gfx950 compute unit
 constexpr int kDenseTileVectors = 300;         // average vectors per tile from which a unit counts as dense (about 85 % sparsity)
@@ -303,14 +305,11 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
     // that it is among them; the number of tokens is the template's.)
     const int W = wave_counts & 0xff, dense_waves = wave_counts >> 8;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    constexpr int VPL = kVecPerLane;
     constexpr int D = kRing;
     constexpr int NTOK = HALF ? 8 : NB * 16;      // tokens
     // activation loads per issue: two fragments per column block, or (ROWMAJ) the tile's
     // 64 x N block as 1 KiB pieces
     constexpr int BL = BLDS ? 0 : (ROWMAJ ? NTOK / 8 : 2 * NB);
-    constexpr int L = VPL + BL;                   // loads per issue: word loads (+ activation loads)
-    constexpr int kSeg = VPL * kWave;             // vectors per segment
 
     static_assert(!(KSPLIT && BLDS), "a workgroup that splits K shares no activation slice");
     static_assert(!(ROWMAJ && BLDS), "row-major activations are not staged");
@@ -329,6 +328,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
     int kb1 = kb0 + avg;
     kb1 = kb1 < nkb ? kb1 : nkb;
     int Wk = W;    // waves that work in a K-splitting workgroup
+    bool long_tiles = false;
     int wreg = 0;  // offsets window: lane l holds the offset of tile wbase + l of this wave's run
     bool cleared = false;
     uint8_t* const tile = lds + wave * kTileBytes;
@@ -381,7 +381,9 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         settle(wreg);
         settle(e0);
         settle(e1);
-        if (adaptive && __builtin_amdgcn_readfirstlane(e1 - e0) >= kDenseTileVectors * n) {
+        const int unit_vectors = __builtin_amdgcn_readfirstlane(e1 - e0);
+        long_tiles = unit_vectors >= kLongTileVectors * n && unit_vectors <= kVecPerLaneLong * kWave * n;
+        if (adaptive && unit_vectors >= kDenseTileVectors * n) {
             Wk = dense_waves;
             b0 = d0;
             b1 = d1;
@@ -465,233 +467,246 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
     }
     // Per-lane byte offsets of the word loads: chunk u sits at lane*16 + u*1024 and the
     // instruction's immediate offset reaches 4095.
-    const int voff_lo = lane * 16, voff_hi = lane * 16 + 4096;
+    const int voff_lo = lane * 16, voff_hi = lane * 16 + 4096, voff_top = lane * 16 + 8192;
     // constants the scatter asm wants in VGPRs
     uint32_t vzero = 0, vtwo = 2, vbase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(tile));
     asm volatile("" : "+v"(vzero), "+v"(vtwo), "+v"(vbase));
 
-    // The unit's stream is cut into segments of up to kSeg vectors that never cross a tile:
-    // a tile of n vectors is ceil(n / kSeg) segments, an empty tile one empty segment.
-    struct Seg {
-        int tile;     // index within the unit; ntile = past the end
-        int begin;    // first vector, absolute
-        int n;        // vectors in this segment
-        bool first;   // first segment of its tile
-        bool last;    // last segment of its tile
-    };
-    struct Cur {
-        int tile, off;
-    };
-    auto make_seg = [&](Cur c, Seg& s, Cur& nxt) {
-        if (c.tile >= ntile) {
-            s = Seg{ntile, 0, 0, true, true};
-            nxt = c;
-            return;
-        }
-        int b, e;
-        tile_range(c.tile, b, e);
-        const int rest = e - b - c.off;
-        s.tile = c.tile;
-        s.begin = b + c.off;
-        s.n = rest < kSeg ? rest : kSeg;
-        s.first = c.off == 0;
-        s.last = rest <= kSeg;
-        nxt = s.last ? Cur{c.tile + 1, 0} : Cur{c.tile, c.off + kSeg};
-    };
-
-    u32x4 regs[D][VPL];
-    half8 bfrag[D][BL > 0 ? BL : 1];  // only used when the activations come from global memory
-    Seg held[D] = {};
-
-    // Always exactly L loads, whatever the segment holds, so the wait counts are static.
-    auto issue = [&](int slot, const Seg& s) {
-        // No more than one full segment's worth (8 KiB) of words in flight per wave: beyond that
-        // the memory system only queues (about 4 % slower on a 165 MB stream at 80 % sparsity,
-        // where two tiles would be 13 KiB).  Two small tiles together (90 % sparsity and up) may
-        // both be in flight, or a wave's 3 KiB at a time would leave it latency bound.
-        if (held[slot ^ 1].n + s.n > kSeg)
-            wait_loads<0>();
-        const bool live = s.tile < ntile;
-        const uint64_t base = reinterpret_cast<uint64_t>(items + s.begin);
-        // descriptor over exactly this segment (nothing at all past the end of the unit)
-        i32x4 rs = {(int)(uint32_t)base, (int)((uint32_t)(base >> 32) & 0xffff), live ? s.n * 16 : 0, 0x00020000};
-        // Activation loads go first: they hit in L2 and return quickly, and loads return in order,
-        // so behind the weight loads they would hold their slots for a full HBM round trip (1-3 %).
-        if (!BLDS) {
-            const int bt = live ? s.tile : ntile - 1;
-            if (ROWMAJ) {
-                // B[k][n]: the tile's 64 x N block is contiguous; piece h = bytes [1024 h, 1024 h + 1024)
-                const _Float16* blk = B + (size_t)(kb0 + bt) * (kTileCols * NTOK);
-#pragma unroll
-                for (int h = 0; h < BL; h++)
-                    bfrag[slot][h] = load_activations_at(blk + h * 512, lane * 16);
-            } else {
-#pragma unroll
-                for (int cb = 0; cb < NB; cb++)
-#pragma unroll
-                    for (int k = 0; k < 2; k++)
-                        bfrag[slot][cb * 2 + k] = load_activations(bptr[cb] + bt * kTileCols + k * 32);
+    // Everything from here to the end of the run is written once for any number VPL of 16-byte
+    // vectors per lane and segment (ring slot), and instantiated for two: kVecPerLane (8: tiles
+    // up to 25 % dense in one segment) and kVecPerLaneLong (10).  A tile that does not fit one
+    // segment costs a full clear of the image instead of an un-scatter, about 14 % of the time
+    // per tile; ten vectors per lane cost 1.3 % on tiles that fit eight.  So a K-splitting
+    // workgroup picks by its own unit's density (long_tiles, set where the density is read).
+    auto stream_run = [&](auto vpl_c) {
+        constexpr int VPL = decltype(vpl_c)::value;
+        constexpr int L = VPL + BL;        // loads per issue: word loads (+ activation loads)
+        constexpr int kSeg = VPL * kWave;  // vectors per segment
+        // The unit's stream is cut into segments of up to kSeg vectors that never cross a tile:
+        // a tile of n vectors is ceil(n / kSeg) segments, an empty tile one empty segment.
+        struct Seg {
+            int tile;     // index within the unit; ntile = past the end
+            int begin;    // first vector, absolute
+            int n;        // vectors in this segment
+            bool first;   // first segment of its tile
+            bool last;    // last segment of its tile
+        };
+        struct Cur {
+            int tile, off;
+        };
+        auto make_seg = [&](Cur c, Seg& s, Cur& nxt) {
+            if (c.tile >= ntile) {
+                s = Seg{ntile, 0, 0, true, true};
+                nxt = c;
+                return;
             }
-        }
-        static_for<VPL>([&](auto uc) {
-            constexpr int u = decltype(uc)::value;
-            if constexpr (u < 4)
-                regs[slot][u] = load_words<u * 1024>(rs, voff_lo);
-            else
-                regs[slot][u] = load_words<(u - 4) * 1024>(rs, voff_hi);
-        });
-    };
+            int b, e;
+            tile_range(c.tile, b, e);
+            const int rest = e - b - c.off;
+            s.tile = c.tile;
+            s.begin = b + c.off;
+            s.n = rest < kSeg ? rest : kSeg;
+            s.first = c.off == 0;
+            s.last = rest <= kSeg;
+            nxt = s.last ? Cur{c.tile + 1, 0} : Cur{c.tile, c.off + kSeg};
+        };
 
-    // Waits for every load of `slot` (at most Y younger ones may stay in flight) and keeps the
-    // slot's registers live up to that point, so none of them can be reused while a load into
-    // it is still on its way.
-    auto land = [&](int slot, auto younger) {
-        constexpr int Y = decltype(younger)::value;
-        wait_loads<Y>();
-        static_for<VPL>([&](auto uc) { pin(regs[slot][decltype(uc)::value]); });
-        if (!BLDS) {
-#pragma unroll
-            for (int h = 0; h < BL; h++)
-                settle(bfrag[slot][h]);
-        }
-    };
+        u32x4 regs[D][VPL];
+        half8 bfrag[D][BL > 0 ? BL : 1];  // only used when the activations come from global memory
+        Seg held[D] = {};
 
-    // Y = loads issued after this slot's that may stay in flight.  The slot's loads were issued
-    // a whole tile ago, so waiting for all of them up front costs nothing in steady state and
-    // keeps one unconditional wait on every path through the loop.
-    auto consume = [&](int slot, const Seg& s, auto younger) {
-        land(slot, younger);
-        if (s.n == 0)
-            return;  // empty tile or past the end
-        constexpr bool kKeep = NB == 1;  // room for the 32 addresses only with one column block
-        uint32_t kept[kKeep ? VPL : 1][4];
-        // One code path per number of full 64-vector chunks (a uniform switch): those run
-        // unguarded, the one partial chunk under a lane mask, the rest not at all.  (A lane mask
-        // per chunk costs a compare and three scalar instructions each, twice per tile.)
-        const int full = s.n >> 6;
-        const bool in_part = (full << 6) + lane < s.n;  // this lane's vector of the partial chunk exists
-        auto by_chunks = [&](auto&& op) {
-            auto run = [&](auto pc) {
-                constexpr int P = decltype(pc)::value;
-                static_for<P>([&](auto uc) { op(uc); });
-                if constexpr (P < VPL) {
-                    if (in_part)
-                        op(pc);
+        // Always exactly L loads, whatever the segment holds, so the wait counts are static.
+        auto issue = [&](int slot, const Seg& s) {
+            // No more than one full segment's worth (8 KiB) of words in flight per wave: beyond that
+            // the memory system only queues (about 4 % slower on a 165 MB stream at 80 % sparsity,
+            // where two tiles would be 13 KiB).  Two small tiles together (90 % sparsity and up) may
+            // both be in flight, or a wave's 3 KiB at a time would leave it latency bound.
+            if (held[slot ^ 1].n + s.n > kSeg)
+                wait_loads<0>();
+            const bool live = s.tile < ntile;
+            const uint64_t base = reinterpret_cast<uint64_t>(items + s.begin);
+            // descriptor over exactly this segment (nothing at all past the end of the unit)
+            i32x4 rs = {(int)(uint32_t)base, (int)((uint32_t)(base >> 32) & 0xffff), live ? s.n * 16 : 0, 0x00020000};
+            // Activation loads go first: they hit in L2 and return quickly, and loads return in order,
+            // so behind the weight loads they would hold their slots for a full HBM round trip (1-3 %).
+            if (!BLDS) {
+                const int bt = live ? s.tile : ntile - 1;
+                if (ROWMAJ) {
+                    // B[k][n]: the tile's 64 x N block is contiguous; piece h = bytes [1024 h, 1024 h + 1024)
+                    const _Float16* blk = B + (size_t)(kb0 + bt) * (kTileCols * NTOK);
+    #pragma unroll
+                    for (int h = 0; h < BL; h++)
+                        bfrag[slot][h] = load_activations_at(blk + h * 512, lane * 16);
+                } else {
+    #pragma unroll
+                    for (int cb = 0; cb < NB; cb++)
+    #pragma unroll
+                        for (int k = 0; k < 2; k++)
+                            bfrag[slot][cb * 2 + k] = load_activations(bptr[cb] + bt * kTileCols + k * 32);
                 }
-            };
-            switch (full) {
-                case 0: run(std::integral_constant<int, 0>{}); break;
-                case 1: run(std::integral_constant<int, 1>{}); break;
-                case 2: run(std::integral_constant<int, 2>{}); break;
-                case 3: run(std::integral_constant<int, 3>{}); break;
-                case 4: run(std::integral_constant<int, 4>{}); break;
-                case 5: run(std::integral_constant<int, 5>{}); break;
-                case 6: run(std::integral_constant<int, 6>{}); break;
-                case 7: run(std::integral_constant<int, 7>{}); break;
-                default: run(std::integral_constant<int, 8>{}); break;
+            }
+            static_for<VPL>([&](auto uc) {
+                constexpr int u = decltype(uc)::value;
+                if constexpr (u < 4)
+                    regs[slot][u] = load_words<u * 1024>(rs, voff_lo);
+                else if constexpr (u < 8)
+                    regs[slot][u] = load_words<(u - 4) * 1024>(rs, voff_hi);
+                else
+                    regs[slot][u] = load_words<(u - 8) * 1024>(rs, voff_top);
+            });
+        };
+
+        // Waits for every load of `slot` (at most Y younger ones may stay in flight) and keeps the
+        // slot's registers live up to that point, so none of them can be reused while a load into
+        // it is still on its way.
+        auto land = [&](int slot, auto younger) {
+            constexpr int Y = decltype(younger)::value;
+            wait_loads<Y>();
+            static_for<VPL>([&](auto uc) { pin(regs[slot][decltype(uc)::value]); });
+            if (!BLDS) {
+    #pragma unroll
+                for (int h = 0; h < BL; h++)
+                    settle(bfrag[slot][h]);
             }
         };
-        static_assert(VPL == 8, "the switch above lists 0..8 full chunks");
-        by_chunks([&](auto uc) {
-            constexpr int u = decltype(uc)::value;
-            if constexpr (kKeep)
-                scatter_words_keep(regs[slot][u], vbase, vtwo, kept[u]);
-            else
-                scatter_words<false>(regs[slot][u], vbase, vtwo, vzero);
-        });
-        if (!s.last)
-            return;  // more segments of this tile follow
-        half8 bf[NB][2];
-        if (BLDS || ROWMAJ) {
-            const uint8_t* bt = bslice + (BLDS ? (size_t)s.tile * (NTOK * 128) : 0);
-            if (ROWMAJ) {
-                // lane l of piece h holds tokens n0 .. n0+7 of row k, (k, n0) = divmod(512 h + 8 l, N);
-                // element (k, n) goes to byte n*128 + (((k >> 3) ^ (n & 7)) << 4) + 2*(k & 7), n & 7 = j
-#pragma unroll
-                for (int h = 0; h < BL; h++) {
-                    const int e0 = h * 512 + lane * 8;
-                    const int k = e0 / NTOK, n0 = e0 % NTOK;
-                    const int base = n0 * 128 + (k & 7) * 2, g0 = (k >> 3) << 4;
-#pragma unroll
-                    for (int j = 0; j < 8; j++)
-                        *reinterpret_cast<_Float16*>(bslice + ((g0 ^ (j << 4)) + base) + j * 128) = bfrag[slot][h][j];
-                }
-            }
-#pragma unroll
-            for (int cb = 0; cb < NB; cb++)
-#pragma unroll
-                for (int k = 0; k < 2; k++)
-                    bf[cb][k] = *reinterpret_cast<const half8*>(bt + b_off[cb][k]);
-        } else {
-#pragma unroll
-            for (int cb = 0; cb < NB; cb++)
-#pragma unroll
-                for (int k = 0; k < 2; k++)
-                    bf[cb][k] = bfrag[slot][cb * 2 + k];
-        }
-        // read the dense tile back and multiply; all reads of a pass are issued before its MFMAs
-        constexpr int kPasses = NB == 1 ? 1 : 2;
-        constexpr int kStepsPerPass = 2 / kPasses;
-#pragma unroll
-        for (int p = 0; p < kPasses; p++) {
-            half8 afrag[kStepsPerPass][8];
-#pragma unroll
-            for (int k = 0; k < kStepsPerPass; k++)
-#pragma unroll
-                for (int r = 0; r < 8; r++)
-                    afrag[k][r] = *reinterpret_cast<const half8*>(tile + a_off[p * kStepsPerPass + k] + r * 2048);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int k = 0; k < kStepsPerPass; k++)
-#pragma unroll
-                for (int r = 0; r < 8; r++)
-#pragma unroll
-                    for (int cb = 0; cb < NB; cb++)
-                        acc[cb][r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[k][r], bf[cb][p * kStepsPerPass + k],
-                                                                            acc[cb][r], 0, 0, 0);
-        }
-        // restore the all-zero tile: undo this segment's writes, or clear everything when
-        // earlier segments (whose words are gone) wrote into it as well
-        if (!s.first) {
-            clear_tile(tile, lane);
-        } else {
+
+        // Y = loads issued after this slot's that may stay in flight.  The slot's loads were issued
+        // a whole tile ago, so waiting for all of them up front costs nothing in steady state and
+        // keeps one unconditional wait on every path through the loop.
+        auto consume = [&](int slot, const Seg& s, auto younger) {
+            land(slot, younger);
+            if (s.n == 0)
+                return;  // empty tile or past the end
+            constexpr bool kKeep = NB == 1;  // room for the 32 addresses only with one column block
+            uint32_t kept[kKeep ? VPL : 1][4];
+            // One code path per number of full 64-vector chunks (a uniform switch): those run
+            // unguarded, the one partial chunk under a lane mask, the rest not at all.  (A lane mask
+            // per chunk costs a compare and three scalar instructions each, twice per tile.)
+            const int full = s.n >> 6;
+            const bool in_part = (full << 6) + lane < s.n;  // this lane's vector of the partial chunk exists
+            auto by_chunks = [&](auto&& op) {
+                auto run = [&](auto pc) {
+                    constexpr int P = decltype(pc)::value;
+                    static_for<P>([&](auto uc) { op(uc); });
+                    if constexpr (P < VPL) {
+                        if (in_part)
+                            op(pc);
+                    }
+                };
+                bool done = false;
+                static_for<VPL + 1>([&](auto pc) {
+                    if (!done && full == decltype(pc)::value) {
+                        run(pc);
+                        done = true;
+                    }
+                });
+            };
             by_chunks([&](auto uc) {
                 constexpr int u = decltype(uc)::value;
                 if constexpr (kKeep)
-                    clear_words(kept[u], vzero);
+                    scatter_words_keep(regs[slot][u], vbase, vtwo, kept[u]);
                 else
-                    scatter_words<true>(regs[slot][u], vbase, vtwo, vzero);
+                    scatter_words<false>(regs[slot][u], vbase, vtwo, vzero);
             });
-        }
-    };
+            if (!s.last)
+                return;  // more segments of this tile follow
+            half8 bf[NB][2];
+            if (BLDS || ROWMAJ) {
+                const uint8_t* bt = bslice + (BLDS ? (size_t)s.tile * (NTOK * 128) : 0);
+                if (ROWMAJ) {
+                    // lane l of piece h holds tokens n0 .. n0+7 of row k, (k, n0) = divmod(512 h + 8 l, N);
+                    // element (k, n) goes to byte n*128 + (((k >> 3) ^ (n & 7)) << 4) + 2*(k & 7), n & 7 = j
+    #pragma unroll
+                    for (int h = 0; h < BL; h++) {
+                        const int e0 = h * 512 + lane * 8;
+                        const int k = e0 / NTOK, n0 = e0 % NTOK;
+                        const int base = n0 * 128 + (k & 7) * 2, g0 = (k >> 3) << 4;
+    #pragma unroll
+                        for (int j = 0; j < 8; j++)
+                            *reinterpret_cast<_Float16*>(bslice + ((g0 ^ (j << 4)) + base) + j * 128) = bfrag[slot][h][j];
+                    }
+                }
+    #pragma unroll
+                for (int cb = 0; cb < NB; cb++)
+    #pragma unroll
+                    for (int k = 0; k < 2; k++)
+                        bf[cb][k] = *reinterpret_cast<const half8*>(bt + b_off[cb][k]);
+            } else {
+    #pragma unroll
+                for (int cb = 0; cb < NB; cb++)
+    #pragma unroll
+                    for (int k = 0; k < 2; k++)
+                        bf[cb][k] = bfrag[slot][cb * 2 + k];
+            }
+            // read the dense tile back and multiply; all reads of a pass are issued before its MFMAs
+            constexpr int kPasses = NB == 1 ? 1 : 2;
+            constexpr int kStepsPerPass = 2 / kPasses;
+    #pragma unroll
+            for (int p = 0; p < kPasses; p++) {
+                half8 afrag[kStepsPerPass][8];
+    #pragma unroll
+                for (int k = 0; k < kStepsPerPass; k++)
+    #pragma unroll
+                    for (int r = 0; r < 8; r++)
+                        afrag[k][r] = *reinterpret_cast<const half8*>(tile + a_off[p * kStepsPerPass + k] + r * 2048);
+                __builtin_amdgcn_sched_barrier(0);
+    #pragma unroll
+                for (int k = 0; k < kStepsPerPass; k++)
+    #pragma unroll
+                    for (int r = 0; r < 8; r++)
+    #pragma unroll
+                        for (int cb = 0; cb < NB; cb++)
+                            acc[cb][r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[k][r], bf[cb][p * kStepsPerPass + k],
+                                                                                acc[cb][r], 0, 0, 0);
+            }
+            // restore the all-zero tile: undo this segment's writes, or clear everything when
+            // earlier segments (whose words are gone) wrote into it as well
+            if (!s.first) {
+                clear_tile(tile, lane);
+            } else {
+                by_chunks([&](auto uc) {
+                    constexpr int u = decltype(uc)::value;
+                    if constexpr (kKeep)
+                        clear_words(kept[u], vzero);
+                    else
+                        scatter_words<true>(regs[slot][u], vbase, vtwo, vzero);
+                });
+            }
+        };
 
-    if (ntile > 0) {
-        Cur ci{0, 0};
-#pragma unroll
-        for (int s = 0; s < D; s++) {
-            Cur nx;
-            make_seg(ci, held[s], nx);
-            ci = nx;
-            issue(s, held[s]);
-        }
-        for (;;) {
-#pragma unroll
+        if (ntile > 0) {
+            Cur ci{0, 0};
+    #pragma unroll
             for (int s = 0; s < D; s++) {
-                consume(s, held[s], std::integral_constant<int, (D - 1) * L>{});
                 Cur nx;
                 make_seg(ci, held[s], nx);
                 ci = nx;
                 issue(s, held[s]);
             }
-            if (held[0].tile >= ntile)
-                break;  // every later slot is past the end as well
+            for (;;) {
+    #pragma unroll
+                for (int s = 0; s < D; s++) {
+                    consume(s, held[s], std::integral_constant<int, (D - 1) * L>{});
+                    Cur nx;
+                    make_seg(ci, held[s], nx);
+                    ci = nx;
+                    issue(s, held[s]);
+                }
+                if (held[0].tile >= ntile)
+                    break;  // every later slot is past the end as well
+            }
+            // the loads of the last (empty) issues are still in flight: let them land while their
+            // destination registers are still reserved
+    #pragma unroll
+            for (int s = 0; s < D; s++)
+                land(s, std::integral_constant<int, 0>{});
         }
-        // the loads of the last (empty) issues are still in flight: let them land while their
-        // destination registers are still reserved
-#pragma unroll
-        for (int s = 0; s < D; s++)
-            land(s, std::integral_constant<int, 0>{});
-    }
+
+    };
+    if (KSPLIT && NB == 1 && long_tiles)
+        stream_run(std::integral_constant<int, kVecPerLaneLong>{});
+    else
+        stream_run(std::integral_constant<int, kVecPerLane>{});
 
     auto write_out = [&]() {
     // Epilogue.  acc[c][r][i] is output row r*16 + 4*q + i of this tile row for token

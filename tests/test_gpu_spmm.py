@@ -667,3 +667,36 @@ def test_every_partition_of_a_tile_row_among_the_waves(spmm, oracle, flags):
                                          waves, 0, 0, flags)
             torch.cuda.synchronize()
             assert np.array_equal(d_C.cpu().numpy(), ref.astype(np.float16)), (tiles, waves)  # integers: exact
+
+
+@pytest.mark.parametrize("N,split_k,waves", [(16, 1, 5), (8, 2, 8), (16, 3, 3)])
+def test_long_segments_follow_each_tile_rows_density(spmm, oracle, N, split_k, waves):
+    """In the K-splitting layout a workgroup whose tiles mostly exceed 512 vectors streams them in
+    segments of 640 instead of 512.  Tile rows alternate between 70 % sparsity (about 614 vectors
+    per tile: the long segments), 80 % (410: the short ones) and 55 % (920: short ones, two per
+    tile), so all three cases run in one launch; a few tiles of the first kind exceed 640 and
+    take two long segments."""
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    M, K = 128 * 9, 64 * 40
+    parts = [spmm.synth_weights(M, K, sp, False, seed=70 + i).view(np.uint16) for i, sp in enumerate((0.7, 0.8, 0.55))]
+    which = (np.arange(M) // 128) % 3
+    A = np.choose(which[:, None], parts).view(np.float16)
+    A[0:128, 0:64] = spmm.synth_weights(128, 64, 0.6, False, seed=77)  # one tile of 820 vectors in a 614-average row
+    B = spmm.synth_activations(N, K, seed=78)
+    items, offsets = spmm.InitSparseMatrixA_API(A)
+    per_tile = np.diff(offsets[:-1]).reshape(M // 128, K // 64)
+    means = per_tile.mean(axis=1)
+    assert 498 <= means[0] <= 640 and means[1] < 498 and means[2] > 640 and per_tile[0].max() > 640
+    ref = oracle.gemm_f32(A, B)
+    d_items = torch.from_numpy(items.view(np.int32).copy()).to(dev)
+    d_offs = torch.from_numpy(offsets.copy()).to(dev)
+    d_B = torch.from_numpy(B.view(np.int16).copy()).to(dev)
+    for flags in (0, 4):
+        d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device=dev)
+        d_W = torch.full((split_k, N, M), float("nan"), dtype=torch.float16, device=dev) if split_k > 1 else None
+        print(f"[gpu case] long segments N={N} split_k={split_k} waves={waves} flags={flags}", flush=True)
+        spmm.SpMM_SplitK_API_Planned(torch.cuda.current_stream(), d_items, d_offs, d_B, d_C, M, N, K, d_W, split_k, 1,
+                                     waves, 0, 0, flags)
+        torch.cuda.synchronize()
+        assert_close(d_C.cpu().numpy(), ref)
