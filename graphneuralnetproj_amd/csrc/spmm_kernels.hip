@@ -703,7 +703,13 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         }
 
     };
-    if (KSPLIT && NB == 1 && long_tiles)
+    if (!KSPLIT && ntile > 0) {
+        // a wave of the row-sharing layout owns its run alone and judges it by its offsets window
+        const int nw = ntile < kWave - 1 ? ntile : kWave - 1;
+        const int run_vectors = __builtin_amdgcn_readlane(wreg, nw) - __builtin_amdgcn_readlane(wreg, 0);
+        long_tiles = run_vectors >= kLongTileVectors * nw && run_vectors <= kVecPerLaneLong * kWave * nw;
+    }
+    if (long_tiles)
         stream_run(std::integral_constant<int, kVecPerLaneLong>{});
     else
         stream_run(std::integral_constant<int, kVecPerLane>{});
