@@ -482,6 +482,13 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         constexpr int VPL = decltype(vpl_c)::value;
         constexpr int L = VPL + BL;        // loads per issue: word loads (+ activation loads)
         constexpr int kSeg = VPL * kWave;  // vectors per segment
+        // Vectors a wave may have in flight.  One full segment's worth (8 KiB): beyond that the
+        // memory system only queues (about 4 % slower on a 165 MB stream at 80 % sparsity with
+        // five and more waves per compute unit, where two tiles would be 13 KiB).  Two segments'
+        // worth where at most four waves work on a compute unit (one per SIMD: fewer requesters,
+        // -0.7 %), except at N = 64.  Two small tiles together (90 % sparsity and up) may always
+        // both be in flight, or a wave's 3 KiB at a time would leave it latency bound.
+        const int flight = NB <= 2 && (KSPLIT ? Wk : W) <= 4 ? 2 * kSeg : kSeg;
         // The unit's stream is cut into segments of up to kSeg vectors that never cross a tile:
         // a tile of n vectors is ceil(n / kSeg) segments, an empty tile one empty segment.
         struct Seg {
@@ -517,11 +524,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
 
         // Always exactly L loads, whatever the segment holds, so the wait counts are static.
         auto issue = [&](int slot, const Seg& s) {
-            // No more than one full segment's worth (8 KiB) of words in flight per wave: beyond that
-            // the memory system only queues (about 4 % slower on a 165 MB stream at 80 % sparsity,
-            // where two tiles would be 13 KiB).  Two small tiles together (90 % sparsity and up) may
-            // both be in flight, or a wave's 3 KiB at a time would leave it latency bound.
-            if (held[slot ^ 1].n + s.n > kSeg)
+            if (held[slot ^ 1].n + s.n > flight)
                 wait_loads<0>();
             const bool live = s.tile < ntile;
             const uint64_t base = reinterpret_cast<uint64_t>(items + s.begin);
