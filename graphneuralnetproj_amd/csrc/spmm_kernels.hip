@@ -74,7 +74,8 @@ constexpr int kVecPerLaneLong = 10;  // ... and for units whose tiles mostly exc
 constexpr int kLongTileVectors = 498;  // average vectors per tile from which a unit takes the long segments
 constexpr int kRing = 2;        // ring slots: one tile being consumed, one in flight
 constexpr unsigned kMaxLdsBytes = 160 * 1024;  // LDS of one gfx950 compute unit
-constexpr int kDenseTileVectors = 300;         // average vectors per tile from which a unit counts as dense (about 85 % sparsity)
+constexpr int kDenseTileVectors = 340;         // average vectors per tile from which a unit counts as dense (about 83 % sparsity)
+constexpr int kSparseWaves = 6;                // waves that work on a sparse unit when the launch shape is adaptive
 
 // Arrival counters of the fused split-K reduction: one page per caller stream, one counter per
 // group of output rows.  Zero when the module is loaded; the workgroup that brings a counter to
@@ -355,17 +356,21 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
             b0 = kb0 + cut(wave);
             b1 = kb0 + cut(wave + 1);
         };
-        int b0, b1;
-        run(W, b0, b1);
-        // The host launches the waves that sparse tiles want (small tiles: a wave's turnaround per
-        // tile, not the memory system, is the limit, so more waves help) and says how many dense
-        // tiles want; the unit's own density decides.  The others stream nothing and wait at the
-        // barrier of the final sum, of which they take their share.  The offsets windows of both
+        // The host launches eight waves and says how many of them dense tiles want; sparse tiles
+        // want kSparseWaves (small tiles: a wave's turnaround per tile, not the memory system, is
+        // the limit, so more waves help, up to a point); the unit's own density decides.  The
+        // others stream nothing and wait at the barrier of the final sum, of which they take
+        // their share.  The offsets windows of both
         // outcomes travel with the two offsets that give the density, so the decision costs no
         // memory round trip of its own.  (All four loads are issued on every path, adaptive or
         // not, and waited for in one place: a value that is still on its way must not meet
         // another at a join, where the compiler would copy it.)
         const bool adaptive = dense_waves > 0 && dense_waves < W && n > 0;
+        const int sparse_waves = adaptive && W > kSparseWaves ? kSparseWaves : W;
+        int b0 = kb0, b1 = kb0;
+        if (wave < sparse_waves)
+            run(sparse_waves, b0, b1);
+        Wk = sparse_waves;
         int d0 = kb0, d1 = kb0;
         if (adaptive && wave < dense_waves)
             run(dense_waves, d0, d1);
@@ -946,7 +951,7 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
 // fuse_page >= 0: out = Split_K dense slabs, and the kernel itself reduces them into fused_out
 // (token stride ldc), counting arrivals on that page of counters; at most 4096 row groups.
 // dense_waves (mode 1; 0 = off): of the `waves` launched, only this many work on a unit whose
-// tiles average 300 vectors or more; the kernel looks at each unit's own offsets.
+// tiles average 340 vectors or more (six on sparser units); the kernel looks at each unit's own offsets.
 extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offsets, const void* B, void* out, int M,
                                 int N, int K, int split_k, int mode, int waves, int stage_b, int row_major,
                                 unsigned lds_bytes, int ldb, int ldo, int relu, void* fused_out, int ldc,
