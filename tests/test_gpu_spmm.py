@@ -700,3 +700,39 @@ def test_long_segments_follow_each_tile_rows_density(spmm, oracle, N, split_k, w
                                      waves, 0, 0, flags)
         torch.cuda.synchronize()
         assert_close(d_C.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("M,K", [(21504, 7168), (7168, 28672), (27648, 9216), (9216, 9216), (36864, 9216), (9216, 36864)])
+def test_benchmark_shapes_with_their_planned_launch(spmm, oracle, M, K):
+    """The other OPT-30B / OPT-66B shapes of the benchmark at full size, each with the Split_K and launch
+    shape the library plans for it, for 8, 16 and 32 tokens: 96 sampled output rows (whole tile rows are
+    too slow for the CPU checker) against the oracle, and every row through linearity in B:
+    C(B1 + B2) = C(B1) + C(B2) within fp16 rounding of the three results."""
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    A = spmm.synth_weights(M, K, 0.8, False, seed=M // 128 + K)
+    items, offsets = spmm.InitSparseMatrixA_API(A)
+    d_items = torch.from_numpy(items.view(np.int32)).to(dev)
+    d_offs = torch.from_numpy(offsets).to(dev)
+    rows = np.sort(np.random.default_rng(M + K).choice(M, size=96, replace=False))
+    A_rows = np.ascontiguousarray(A[rows])
+    for N in (8, 16, 32):
+        split_k = spmm.SpMM_SuggestSplitK(M, N, K)
+        B1 = spmm.synth_activations(N, K, seed=5 + N)
+        B2 = spmm.synth_activations(N, K, seed=6 + N)
+        B3 = (B1.astype(np.float32) + B2.astype(np.float32)).astype(np.float16)
+        outs = []
+        d_W = torch.zeros((max(split_k, 1), N, M), dtype=torch.float16, device=dev)
+        for Bx in (B1, B2, B3):
+            d_B = torch.from_numpy(Bx.view(np.int16).copy()).to(dev)
+            d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device=dev)
+            print(f"[gpu case] benchmark shape M={M} K={K} N={N} split_k={split_k}", flush=True)
+            spmm.SpMM_SplitK_API(torch.cuda.current_stream(), None, d_items, d_offs, d_B, d_C, M, N, K, d_W, split_k)
+            torch.cuda.synchronize()
+            outs.append(d_C.cpu().numpy().astype(np.float32))
+        assert_close(outs[0][:, rows], oracle.gemm_f32(A_rows, B1))
+        # B3 is B1 + B2 rounded to fp16: compare against the sum within the tolerance of each term
+        # plus the effect of that rounding (2^-11 relative on every input of a sum of K * 0.2 terms)
+        lin = np.abs(outs[2] - (outs[0] + outs[1]))
+        bound = 3 * (ATOL + RTOL * np.maximum(np.abs(outs[2]), np.abs(outs[0]) + np.abs(outs[1])))
+        assert (lin <= bound).all(), float(lin.max())
