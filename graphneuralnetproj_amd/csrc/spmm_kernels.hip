@@ -178,28 +178,11 @@ __device__ __forceinline__ void pin(const T& x)
     asm volatile("" ::"v"(x));
 }
 
-// Four packed words -> four 16-bit LDS writes of the value (or of zero) at byte
-// address base + 2 * (word >> 16).  One v_mad_u32_u16 on the word's high half forms
-// each address; all four are formed first so the writes issue back to back.
+// Four packed words -> four 16-bit LDS writes of the value at byte address
+// base + 2 * (word >> 16).  One v_mad_u32_u16 on the word's high half forms each address;
+// all four are formed first so the writes issue back to back.  The addresses are kept for
+// clear_words, which writes zero to them after the tile has been multiplied.
 #define TCSL_ADDR(d, s) "v_mad_u32_u16 " d ", " s ", %9, %8 op_sel:[1,0,0,0]\n"
-template<bool CLEAR>
-__device__ __forceinline__ void scatter_words(u32x4 w, uint32_t base, uint32_t two, uint32_t zero)
-{
-    uint32_t a0, a1, a2, a3;
-    if (!CLEAR)
-        asm volatile(TCSL_ADDR("%0", "%4") TCSL_ADDR("%1", "%5") TCSL_ADDR("%2", "%6") TCSL_ADDR("%3", "%7")
-                     "ds_write_b16 %0, %4\n ds_write_b16 %1, %5\n ds_write_b16 %2, %6\n ds_write_b16 %3, %7\n"
-                     : "=&v"(a0), "=&v"(a1), "=&v"(a2), "=&v"(a3)
-                     : "v"(w.x), "v"(w.y), "v"(w.z), "v"(w.w), "v"(base), "v"(two)
-                     : "memory");
-    else
-        asm volatile(TCSL_ADDR("%0", "%4") TCSL_ADDR("%1", "%5") TCSL_ADDR("%2", "%6") TCSL_ADDR("%3", "%7")
-                     "ds_write_b16 %0, %10\n ds_write_b16 %1, %10\n ds_write_b16 %2, %10\n ds_write_b16 %3, %10\n"
-                     : "=&v"(a0), "=&v"(a1), "=&v"(a2), "=&v"(a3)
-                     : "v"(w.x), "v"(w.y), "v"(w.z), "v"(w.w), "v"(base), "v"(two), "v"(zero)
-                     : "memory");
-}
-// The same, keeping the four addresses (and, below, writing zero to kept addresses).
 __device__ __forceinline__ void scatter_words_keep(u32x4 w, uint32_t base, uint32_t two, uint32_t (&a)[4])
 {
     asm volatile(TCSL_ADDR("%0", "%4") TCSL_ADDR("%1", "%5") TCSL_ADDR("%2", "%6") TCSL_ADDR("%3", "%7")
@@ -585,8 +568,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
             land(slot, younger);
             if (s.n == 0)
                 return;  // empty tile or past the end
-            constexpr bool kKeep = NB == 1;  // room for the 32 addresses only with one column block
-            uint32_t kept[kKeep ? VPL : 1][4];
+            uint32_t kept[VPL][4];  // the scatter's LDS addresses, for the un-scatter
             // One code path per number of full 64-vector chunks (a uniform switch): those run
             // unguarded, the one partial chunk under a lane mask, the rest not at all.  (A lane mask
             // per chunk costs a compare and three scalar instructions each, twice per tile.)
@@ -611,10 +593,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
             };
             by_chunks([&](auto uc) {
                 constexpr int u = decltype(uc)::value;
-                if constexpr (kKeep)
-                    scatter_words_keep(regs[slot][u], vbase, vtwo, kept[u]);
-                else
-                    scatter_words<false>(regs[slot][u], vbase, vtwo, vzero);
+                scatter_words_keep(regs[slot][u], vbase, vtwo, kept[u]);
             });
             if (!s.last)
                 return;  // more segments of this tile follow
@@ -674,10 +653,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
             } else {
                 by_chunks([&](auto uc) {
                     constexpr int u = decltype(uc)::value;
-                    if constexpr (kKeep)
-                        clear_words(kept[u], vzero);
-                    else
-                        scatter_words<true>(regs[slot][u], vbase, vtwo, vzero);
+                    clear_words(kept[u], vzero);
                 });
             }
         };
