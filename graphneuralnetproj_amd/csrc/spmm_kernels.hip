@@ -29,7 +29,7 @@
 //     back as MFMA operands with ds_read_b128, issues v_mfma_f32_16x16x32_f16 against the
 //     activation fragments (from the staged slice, or fetched from global memory, where they
 //     are L2 resident), and then restores the zeros by writing 0 to the same addresses (kept
-//     in registers where there is room: a wave is busy about 1 us per tile, which five waves
+//     in registers: a wave is busy about 1 us per tile, which five waves
 //     per compute unit only just turn into more than the memory delivers, so every vector
 //     instruction saved shows).  Undoing ~26 scatter instructions is cheaper than re-clearing
 //     16 KiB, which costs as much LDS bandwidth as reading the tile.  The words of a tile may come in any
