@@ -18,7 +18,9 @@ import time
 import numpy as np
 
 OPT_SHAPES = ("28672x7168,7168x28672,21504x7168,7168x7168,27648x9216,9216x9216,36864x9216,9216x36864,"
-              "36864x12288,12288x12288,49152x12288,12288x49152")  # OPT-30B, 66B and 175B on one GPU
+              "36864x12288,12288x12288,49152x12288,12288x49152,"  # OPT-30B, 66B and 175B on one GPU
+              "10752x7168,7168x3584,14336x7168,7168x14336,5376x7168,7168x1792,"  # one GPU's share of OPT-30B on 2 and 4
+              "13824x9216,9216x4608,18432x9216,9216x18432,6912x9216,9216x2304")  # ... and of OPT-66B
 
 
 def candidate_plans(N, tiles_k):
