@@ -167,6 +167,11 @@ LaunchPlan plan_launch(int M, int N, int K, int split_k, bool row_major, double*
                 // cost model's own preference among wave counts is not that sharp.
                 if (mode == 1 && w != 4)
                     continue;
+                // The row-sharing layout is only considered in the shapes the tuner measures and
+                // the constants were fitted on: staged slice and 5..8 waves up to 16 tokens,
+                // fragments from memory and 1, 2 or 4 waves above.
+                if (mode == 0 && (N <= 16 ? (!stage || w < 5) : (stage || (w != 1 && w != 2 && w != 4))))
+                    continue;
                 LaunchPlan p{mode, w, stage, 0};
                 if (!complete_plan(N, K, split_k, row_major, p))
                     continue;
