@@ -70,8 +70,21 @@ constexpr int kTileCols = 64;   // columns of one encoded tile
 constexpr int kTileBytes = kTileRows * kTileCols * 2;
 constexpr int kWave = 64;
 constexpr int kVecPerLane = 8;       // 16-byte vectors per lane and ring slot: 512 vectors, i.e. tiles up to 25 % dense in one go
-constexpr int kVecPerLaneLong = 10;  // ... and for units whose tiles mostly exceed that: 640 vectors, 31 % dense
-constexpr int kLongTileVectors = 498;  // average vectors per tile from which a unit takes the long segments
+// ... and for runs whose tiles are mostly larger or much smaller, picked by the run's average
+// vectors per tile: 10 per lane (640 vectors, 31 % dense) from 498 up to 640, 4 (256) up to 232,
+// 2 (128) up to 112.
+constexpr int kVecPerLaneLong = 10, kVecPerLaneShort = 4, kVecPerLaneTiny = 2;
+constexpr int kLongTileVectors = 498, kShortTileVectors = 232, kTinyTileVectors = 112;
+__device__ __forceinline__ int segment_choice(int vectors, int tiles)  // 0 tiny, 1 short, 2 regular, 3 long
+{
+    if (tiles <= 0)
+        return 2;
+    if (vectors <= kTinyTileVectors * tiles)
+        return 0;
+    if (vectors <= kShortTileVectors * tiles)
+        return 1;
+    return vectors >= kLongTileVectors * tiles && vectors <= kVecPerLaneLong * kWave * tiles ? 3 : 2;
+}
 constexpr int kRing = 2;        // ring slots: one tile being consumed, one in flight
 constexpr unsigned kMaxLdsBytes = 160 * 1024;  // LDS of one gfx950 compute unit
 constexpr int kDenseTileVectors = 340;         // average vectors per tile from which a unit counts as dense (about 83 % sparsity)
@@ -312,7 +325,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
     int kb1 = kb0 + avg;
     kb1 = kb1 < nkb ? kb1 : nkb;
     int Wk = W;    // waves that work in a K-splitting workgroup
-    bool long_tiles = false;
+    int segments = 2;  // segment_choice of this run
     int wreg = 0;  // offsets window: lane l holds the offset of tile wbase + l of this wave's run
     bool cleared = false;
     uint8_t* const tile = lds + wave * kTileBytes;
@@ -370,7 +383,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         settle(e0);
         settle(e1);
         const int unit_vectors = __builtin_amdgcn_readfirstlane(e1 - e0);
-        long_tiles = unit_vectors >= kLongTileVectors * n && unit_vectors <= kVecPerLaneLong * kWave * n;
+        segments = segment_choice(unit_vectors, n);
         if (adaptive && unit_vectors >= kDenseTileVectors * n) {
             Wk = dense_waves;
             b0 = d0;
@@ -461,22 +474,25 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
     asm volatile("" : "+v"(vzero), "+v"(vtwo), "+v"(vbase));
 
     // Everything from here to the end of the run is written once for any number VPL of 16-byte
-    // vectors per lane and segment (ring slot), and instantiated for two: kVecPerLane (8: tiles
-    // up to 25 % dense in one segment) and kVecPerLaneLong (10).  A tile that does not fit one
-    // segment costs a full clear of the image instead of an un-scatter, about 14 % of the time
-    // per tile; ten vectors per lane cost 1.3 % on tiles that fit eight.  So a K-splitting
-    // workgroup picks by its own unit's density (long_tiles, set where the density is read).
+    // vectors per lane and segment (ring slot), and instantiated for four: kVecPerLane (8: tiles
+    // up to 25 % dense in one segment), kVecPerLaneLong (10), kVecPerLaneShort (4) and
+    // kVecPerLaneTiny (2).  A tile that does not fit one segment costs a full clear of the image
+    // instead of an un-scatter, about 14 % of the time per tile; ten vectors per lane cost 1.3 %
+    // on tiles that fit eight; and every issue is VPL load instructions however little a tile
+    // holds, which on small tiles (90 % sparsity and up) is 5 to 14 % of the time.  So a
+    // workgroup (or, in the row-sharing layout, a wave) picks by its own run's density
+    // (`segments`, set where the density is read).
     auto stream_run = [&](auto vpl_c) {
         constexpr int VPL = decltype(vpl_c)::value;
         constexpr int L = VPL + BL;        // loads per issue: word loads (+ activation loads)
         constexpr int kSeg = VPL * kWave;  // vectors per segment
-        // Vectors a wave may have in flight.  One full segment's worth (8 KiB): beyond that the
+        // Vectors a wave may have in flight.  One regular segment's worth (8 KiB): beyond that the
         // memory system only queues (about 4 % slower on a 165 MB stream at 80 % sparsity with
         // five and more waves per compute unit, where two tiles would be 13 KiB).  Two segments'
         // worth where at most four waves work on a compute unit (one per SIMD: fewer requesters,
         // -0.7 %), except at N = 64.  Two small tiles together (90 % sparsity and up) may always
         // both be in flight, or a wave's 3 KiB at a time would leave it latency bound.
-        const int flight = NB <= 2 && (KSPLIT ? Wk : W) <= 4 ? 2 * kSeg : kSeg;
+        const int flight = (NB <= 2 && (KSPLIT ? Wk : W) <= 4 ? 2 : 1) * kVecPerLane * kWave;
         // The unit's stream is cut into segments of up to kSeg vectors that never cross a tile:
         // a tile of n vectors is ceil(n / kSeg) segments, an empty tile one empty segment.
         struct Seg {
@@ -691,10 +707,14 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         // a wave of the row-sharing layout owns its run alone and judges it by its offsets window
         const int nw = ntile < kWave - 1 ? ntile : kWave - 1;
         const int run_vectors = __builtin_amdgcn_readlane(wreg, nw) - __builtin_amdgcn_readlane(wreg, 0);
-        long_tiles = run_vectors >= kLongTileVectors * nw && run_vectors <= kVecPerLaneLong * kWave * nw;
+        segments = segment_choice(run_vectors, nw);
     }
-    if (long_tiles)
+    if (segments == 3)
         stream_run(std::integral_constant<int, kVecPerLaneLong>{});
+    else if (segments == 1)
+        stream_run(std::integral_constant<int, kVecPerLaneShort>{});
+    else if (segments == 0)
+        stream_run(std::integral_constant<int, kVecPerLaneTiny>{});
     else
         stream_run(std::integral_constant<int, kVecPerLane>{});
 

@@ -736,3 +736,37 @@ def test_benchmark_shapes_with_their_planned_launch(spmm, oracle, M, K):
         lin = np.abs(outs[2] - (outs[0] + outs[1]))
         bound = 3 * (ATOL + RTOL * np.maximum(np.abs(outs[2]), np.abs(outs[0]) + np.abs(outs[1])))
         assert (lin <= bound).all(), float(lin.max())
+
+
+@pytest.mark.parametrize("N,split_k,mode,waves,stage_b", [(16, 1, 1, 5, 0), (8, 2, 1, 8, 0), (32, 1, 1, 4, 0), (64, 2, 1, 4, 0),
+                                                         (16, 4, 0, 6, 1), (32, 2, 0, 4, 0)])
+def test_short_segments_on_sparse_tile_rows(spmm, oracle, N, split_k, mode, waves, stage_b):
+    """Runs whose tiles average at most 232 (112) vectors are streamed in segments of 256 (128)
+    vectors.  Tile rows alternate between 90 % sparsity (205 vectors per tile), 96 % (82) and 80 %
+    (410, the regular segments); one 80 % tile sits in a 96 % row and takes four of its row's short
+    segments, and one tile of that row is empty."""
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    M, K = 128 * 9, 64 * 40
+    parts = [spmm.synth_weights(M, K, sp, False, seed=90 + i).view(np.uint16) for i, sp in enumerate((0.9, 0.96, 0.8))]
+    which = (np.arange(M) // 128) % 3
+    A = np.choose(which[:, None], parts).view(np.float16).copy()
+    A[128:256, 64:128] = spmm.synth_weights(128, 64, 0.8, False, seed=97)
+    A[128:256, 192:256] = 0
+    B = spmm.synth_activations(N, K, seed=98)
+    items, offsets = spmm.InitSparseMatrixA_API(A)
+    per_tile = np.diff(offsets[:-1]).reshape(M // 128, K // 64)
+    means = per_tile.mean(axis=1)
+    assert 112 < means[0] <= 232 and means[1] <= 112 and means[2] > 232 and per_tile[1].max() > 384 and per_tile[1].min() == 0
+    ref = oracle.gemm_f32(A, B)
+    d_items = torch.from_numpy(items.view(np.int32).copy()).to(dev)
+    d_offs = torch.from_numpy(offsets.copy()).to(dev)
+    d_B = torch.from_numpy(B.view(np.int16).copy()).to(dev)
+    for flags in ((0, 4) if mode == 1 and N <= 32 else (0,)):
+        d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device=dev)
+        d_W = torch.full((split_k, N, M), float("nan"), dtype=torch.float16, device=dev) if split_k > 1 else None
+        print(f"[gpu case] short segments N={N} split_k={split_k} mode={mode} waves={waves} flags={flags}", flush=True)
+        spmm.SpMM_SplitK_API_Planned(torch.cuda.current_stream(), d_items, d_offs, d_B, d_C, M, N, K, d_W, split_k, mode,
+                                     waves, stage_b, 0, flags)
+        torch.cuda.synchronize()
+        assert_close(d_C.cpu().numpy(), ref)
