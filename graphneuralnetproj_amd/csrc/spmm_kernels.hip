@@ -21,24 +21,28 @@
 //     128-bit buffer loads into a ring of two register slots, a full tile ahead of their
 //     use.  The loads are inline assembly and their completion is awaited with hand-placed
 //     s_waitcnt vmcnt(N): every issue puts a fixed number of loads in flight, so N is a
-//     compile-time constant.  A wave keeps one tile in flight: every wave of the chip doing
-//     so already saturates the memory system, and more only lengthens its queues.
+//     compile-time constant.  A wave keeps 8 KiB of words in flight (16 KiB where at most four
+//     waves work on a compute unit): more only lengthens the memory system's queues.  The
+//     loop is instantiated for 2, 4, 8 and 10 vectors per lane and issue, and a run takes the
+//     one that fits its tiles' size.
 //   * A private 16 KiB LDS tile holds the dense 128x64 fp16 image.  It is cleared once; per
 //     tile the wave scatters the values with ds_write_b16 at byte address 2*index (the index
 //     already carries the XOR swizzle that makes the read-back conflict free), reads the tile
 //     back as MFMA operands with ds_read_b128, issues v_mfma_f32_16x16x32_f16 against the
 //     activation fragments (from the staged slice, or fetched from global memory, where they
 //     are L2 resident), and then restores the zeros by writing 0 to the same addresses (kept
-//     in registers: a wave is busy about 1 us per tile, which five waves
-//     per compute unit only just turn into more than the memory delivers, so every vector
-//     instruction saved shows).  Undoing ~26 scatter instructions is cheaper than re-clearing
-//     16 KiB, which costs as much LDS bandwidth as reading the tile.  The words of a tile may come in any
-//     order (the reference's encoder orders them to spread LDS banks; the kernel is memory
-//     bound either way).
+//     in registers: a wave is busy 0.8 to 1 us per tile, which four or five waves per compute
+//     unit only just turn into more than the memory delivers, so every instruction saved
+//     shows).  Undoing ~26 scatter instructions is cheaper than re-clearing 16 KiB, which costs
+//     as much LDS bandwidth as reading the tile.  The words of a tile may come in any order
+//     (the reference's encoder orders them to spread LDS banks, which is worth 3 % here).
 //   * TileOffsets of the unit sit in one VGPR (lane i = offset i) and are read with
 //     v_readlane, so the steady-state loop performs no scalar memory reads.
 //   * fp32 accumulators stay in registers over the whole run; the epilogue rounds to fp16
-//     once.  Split_K > 1 writes slabs of partial sums; in the runs layout the last workgroup
+//     once.  In the runs layout the host launches eight waves and each workgroup decides from
+//     its own tile row's density how many of them stream (the plan's number on dense rows,
+//     six on sparse ones); all eight share the final sum.
+//   * Split_K > 1 writes slabs of partial sums; in the runs layout the last workgroup
 //     to finish a tile row then adds the slabs up itself (arrival counters in a static device
 //     array, slabs written through and read at system scope), otherwise a second kernel does.
 //   * ROWMAJ takes B as [K][N] and writes [M][N]; strides (ldb, ldo, ldc) and a fused clamp
