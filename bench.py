@@ -167,7 +167,8 @@ def main():
     d_items = [torch.from_numpy(items.view(np.int32)).to(dev)]
     for _ in range(copies - 1):
         d_items.append(d_items[0].clone())
-    d_offs = torch.from_numpy(offsets).to(dev)
+    # every weight copy has its own TileOffsets array, as every layer of a model would
+    d_offs = [torch.from_numpy(offsets).to(dev) for _ in range(copies)]
     d_B = torch.from_numpy(B.view(np.int16)).to(dev)
     d_C = torch.zeros((N, M), dtype=torch.float16, device=dev)
     d_W = torch.zeros((max(split_k, 1), N, M), dtype=torch.float16, device=dev)
@@ -177,10 +178,11 @@ def main():
     stream = torch.cuda.current_stream()
     sptr = ctypes.c_void_p(stream.cuda_stream)
     p_items = [ctypes.c_void_p(t.data_ptr()) for t in d_items]
-    p_offs, p_B, p_C, p_W = (ctypes.c_void_p(t.data_ptr()) for t in (d_offs, d_B, d_C, d_W))
+    p_offs = [ctypes.c_void_p(t.data_ptr()) for t in d_offs]
+    p_B, p_C, p_W = (ctypes.c_void_p(t.data_ptr()) for t in (d_B, d_C, d_W))
 
     def step(i):
-        rc = lib.SpMM_SplitK_API(sptr, None, p_items[i % copies], p_offs, p_B, p_C, M, N, K, p_W, split_k)
+        rc = lib.SpMM_SplitK_API(sptr, None, p_items[i % copies], p_offs[i % copies], p_B, p_C, M, N, K, p_W, split_k)
         if rc:
             raise RuntimeError(f"SpMM_SplitK_API -> {rc}")
 
@@ -217,11 +219,11 @@ def main():
     # bracketed by two HIP events recorded on the launch stream; the average includes the
     # dispatch gap between consecutive kernels but no per-launch event overhead.
     for i in range(min(args.warmup, 200)):
-        lib.SpMM_SplitK_Partials(sptr, p_items[i % copies], p_offs, p_B, p_W, M, N, K, split_k)
+        lib.SpMM_SplitK_Partials(sptr, p_items[i % copies], p_offs[i % copies], p_B, p_W, M, N, K, split_k)
     ev0, ev1 = lib.SpMM_EventCreate(), lib.SpMM_EventCreate()
     lib.SpMM_EventRecord(ev0, sptr)
     for i in range(args.steps):
-        rc = lib.SpMM_SplitK_Partials(sptr, p_items[i % copies], p_offs, p_B, p_W, M, N, K, split_k)
+        rc = lib.SpMM_SplitK_Partials(sptr, p_items[i % copies], p_offs[i % copies], p_B, p_W, M, N, K, split_k)
         if rc:
             raise RuntimeError(f"SpMM_SplitK_Partials -> {rc}")
     lib.SpMM_EventRecord(ev1, sptr)
