@@ -1,0 +1,301 @@
+// gfx950 kernel for the 2:4 part of a weight: C[n][m] (+ split-K slabs) = A1 * B with A1 held as
+// records in sparse-MFMA operand order (layout: a24_format.h).  The reference runs this part on
+// NVIDIA's mma.sp (csrc/SpMM_Kernel.cuh:293-735 with csrc/MMA_PTX.cuh:195-210); nothing of that
+// is reused.  Here a wave loads values and positions straight into the registers that
+// v_smfmac_f32_16x16x32_f16 reads -- no LDS staging, no scatter -- and the activation fragments
+// come from the L2 in the same operand order as in the Tiled-CSL kernel.
+//
+// Work split: a workgroup owns RB consecutive 16-row blocks of one split-K batch; its W waves
+// cut the batch's 128-column units among themselves, keep RB x N/16 accumulator tiles each, and
+// add them up through LDS in wave order at the end (fp32, one rounding to fp16).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <mutex>
+
+namespace {
+
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+constexpr int kRecordBytes = 2304;
+
+struct AFrag {      // one record's share of a lane
+    u32x4 v[2];     // steps 0,1 and steps 2,3: four fp16 values each
+    unsigned idx;   // byte s = positions for step s
+};
+
+template<int NT>
+struct BFrag {
+    half8 b[NT][4];  // token block x step: eight consecutive columns of one token
+};
+
+__device__ __forceinline__ AFrag load_a(const uint8_t* rec, int lane)
+{
+    AFrag a;
+    a.v[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(rec + lane * 16));
+    a.v[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(rec + 1024 + lane * 16));
+    a.idx = __builtin_nontemporal_load(reinterpret_cast<const unsigned*>(rec + 2048 + lane * 4));
+    return a;
+}
+
+template<int NT>
+__device__ __forceinline__ void load_b(BFrag<NT>& f, const _Float16* const (&tok)[NT], int unit)
+{
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+            f.b[t][s] = *reinterpret_cast<const half8*>(tok[t] + (size_t)unit * 128 + s * 32);
+}
+
+__device__ __forceinline__ half4 step_values(const AFrag& a, int s)
+{
+    union {
+        u32x4 u;
+        half4 h[2];
+    } x;
+    x.u = a.v[s >> 1];
+    return x.h[s & 1];
+}
+
+template<int NT, int RB>
+__device__ __forceinline__ void multiply(float4v (&acc)[RB][NT], const AFrag (&a)[RB], const BFrag<NT>& f)
+{
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+#pragma unroll
+        for (int r = 0; r < RB; r++) {
+            acc[r][t] = __builtin_amdgcn_smfmac_f32_16x16x32_f16(step_values(a[r], 0), f.b[t][0], acc[r][t], (int)a[r].idx, 0, 0);
+            acc[r][t] = __builtin_amdgcn_smfmac_f32_16x16x32_f16(step_values(a[r], 1), f.b[t][1], acc[r][t], (int)a[r].idx, 0, 1);
+            acc[r][t] = __builtin_amdgcn_smfmac_f32_16x16x32_f16(step_values(a[r], 2), f.b[t][2], acc[r][t], (int)a[r].idx, 0, 2);
+            acc[r][t] = __builtin_amdgcn_smfmac_f32_16x16x32_f16(step_values(a[r], 3), f.b[t][3], acc[r][t], (int)a[r].idx, 0, 3);
+        }
+    }
+}
+
+// grid (M / (16 * RB), Split_K), block W * 64.  out + batch * slab is the batch's fp16 [N][ldo]
+// result.  n_tokens may be 8 with NT = 1: tokens 8..15 then read token 7 again and are not stored.
+template<int NT, int RB, int W>
+__global__ __launch_bounds__(W* kWave) void a24_spmm_kernel(const uint8_t* __restrict__ packed,
+                                                            const _Float16* __restrict__ B, _Float16* __restrict__ out,
+                                                            int units, int units_per_batch, long ldb, long ldo,
+                                                            long slab, int n_tokens)
+{
+    extern __shared__ float4v lds[];  // [W][RB][NT][64]
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int batch = blockIdx.y;
+    // this wave's units of the batch
+    const int b0 = batch * units_per_batch;
+    const int bcnt = min(units_per_batch, units - b0);
+    const int base = bcnt / W, rem = bcnt % W;
+    const int u0 = b0 + wave * base + min(wave, rem);
+    const int u1 = u0 + base + (wave < rem ? 1 : 0);
+
+    const uint8_t* rec[RB];
+#pragma unroll
+    for (int r = 0; r < RB; r++)
+        rec[r] = packed + ((size_t)(blockIdx.x * RB + r) * units) * kRecordBytes;
+    const _Float16* tok[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        int n = t * 16 + (lane & 15);
+        n = n < n_tokens ? n : n_tokens - 1;
+        tok[t] = B + (size_t)n * ldb + (lane >> 4) * 8;
+    }
+
+    float4v acc[RB][NT];
+#pragma unroll
+    for (int r = 0; r < RB; r++)
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+            acc[r][t] = float4v{0.f, 0.f, 0.f, 0.f};
+
+    AFrag a0[RB], a1[RB];
+    BFrag<NT> f0, f1;
+    int u = u0;
+    if (u < u1) {
+        load_b<NT>(f0, tok, u);
+#pragma unroll
+        for (int r = 0; r < RB; r++)
+            a0[r] = load_a(rec[r] + (size_t)u * kRecordBytes, lane);
+        while (true) {
+            if (u + 1 < u1) {
+                load_b<NT>(f1, tok, u + 1);
+#pragma unroll
+                for (int r = 0; r < RB; r++)
+                    a1[r] = load_a(rec[r] + (size_t)(u + 1) * kRecordBytes, lane);
+            }
+            multiply<NT, RB>(acc, a0, f0);
+            if (++u >= u1)
+                break;
+            if (u + 1 < u1) {
+                load_b<NT>(f0, tok, u + 1);
+#pragma unroll
+                for (int r = 0; r < RB; r++)
+                    a0[r] = load_a(rec[r] + (size_t)(u + 1) * kRecordBytes, lane);
+            }
+            multiply<NT, RB>(acc, a1, f1);
+            if (++u >= u1)
+                break;
+        }
+    }
+
+    // sum over the workgroup's waves, in wave order
+    if constexpr (W > 1) {
+#pragma unroll
+        for (int r = 0; r < RB; r++)
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+                lds[((wave * RB + r) * NT + t) * kWave + lane] = acc[r][t];
+        __syncthreads();
+    }
+    _Float16* dst = out + (size_t)batch * slab;
+    const int row0 = blockIdx.x * RB * 16 + (lane >> 4) * 4;
+    for (int p = wave; p < RB * NT; p += W) {
+        const int r = p / NT, t = p % NT;
+        float4v s;
+        if constexpr (W > 1) {
+            s = lds[(r * NT + t) * kWave + lane];
+            for (int w = 1; w < W; w++) {
+                const float4v x = lds[((w * RB + r) * NT + t) * kWave + lane];
+                s += x;
+            }
+        } else {
+            // with one wave the loop index is compile-time only through this unrolled search
+            s = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int rr = 0; rr < RB; rr++)
+#pragma unroll
+                for (int tt = 0; tt < NT; tt++)
+                    if (rr == r && tt == t)
+                        s = acc[rr][tt];
+        }
+        const int n = t * 16 + (lane & 15);
+        if (n < n_tokens) {
+            half4 h = {static_cast<_Float16>(s[0]), static_cast<_Float16>(s[1]), static_cast<_Float16>(s[2]),
+                       static_cast<_Float16>(s[3])};
+            *reinterpret_cast<half4*>(dst + (size_t)n * ldo + row0 + r * 16) = h;
+        }
+    }
+}
+
+template<int NT, int RB, int W>
+int launch(hipStream_t stream, const void* packed, const void* B, void* out, int M, int N, int K, int split_k, long ldb,
+           long ldo, long slab)
+{
+    const int units = K / 128;
+    const int per_batch = (units + split_k - 1) / split_k;
+    const unsigned lds = W > 1 ? W * RB * NT * kWave * sizeof(float4v) : 0;
+    auto kern = a24_spmm_kernel<NT, RB, W>;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess)
+            return static_cast<int>(e);
+    }
+    hipLaunchKernelGGL(kern, dim3(M / (16 * RB), split_k), dim3(W * kWave), lds, stream,
+                       static_cast<const uint8_t*>(packed), static_cast<const _Float16*>(B), static_cast<_Float16*>(out),
+                       units, per_batch, ldb, ldo, slab, N);
+    return static_cast<int>(hipGetLastError());
+}
+
+template<int NT>
+int launch_nt(hipStream_t s, const void* packed, const void* B, void* out, int M, int N, int K, int split_k, int rb, int waves,
+              long ldb, long ldo, long slab)
+{
+#define A24_CASE(RB_, W_)                  \
+    if (rb == RB_ && waves == W_)          \
+        return launch<NT, RB_, W_>(s, packed, B, out, M, N, K, split_k, ldb, ldo, slab);
+    A24_CASE(1, 4) A24_CASE(1, 8) A24_CASE(2, 2) A24_CASE(2, 4) A24_CASE(2, 8) A24_CASE(4, 1) A24_CASE(4, 2) A24_CASE(4, 4)
+    if constexpr (NT <= 2) {  // larger accumulator sets would not fit the register file
+        A24_CASE(4, 8) A24_CASE(8, 1) A24_CASE(8, 2) A24_CASE(8, 4)
+    }
+#undef A24_CASE
+    return static_cast<int>(hipErrorInvalidValue);
+}
+
+}  // namespace
+
+// Batch b of ceil((K/128)/split_k) units writes fp16 [N][ldo] to out + b * slab.  The caller has
+// checked: M % (16 * rb) == 0, K % 128 == 0, N in {8, 16, 32, 64}, no batch empty, pointers set.
+extern "C" int a24_launch_spmm(void* stream, const void* packed, const void* B, void* out, int M, int N, int K,
+                               int split_k, int rb, int waves, long ldb, long ldo, long slab)
+{
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (N) {
+        case 8:
+        case 16: return launch_nt<1>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab);
+        case 32: return launch_nt<2>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab);
+        case 64: return launch_nt<4>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab);
+        default: return static_cast<int>(hipErrorInvalidValue);
+    }
+}
+
+// A second stream per caller stream, so that the residual's Tiled-CSL kernel can run beside the 2:4
+// kernel (the reference gives them two streams as well, kernel_benchmark/spmm_test.cu:459-461).
+// Default priority, created on first use, kept until the process ends; at most 32 caller
+// streams get one, further ones run everything on the caller's stream (*side = stream).
+namespace {
+struct SideStream {
+    hipStream_t owner, side;
+    hipEvent_t fork, join;
+};
+std::mutex side_mu;
+SideStream side_table[32];
+int side_used = 0;
+}  // namespace
+
+// Everything enqueued on `stream` so far happens before what is then enqueued on *side.
+extern "C" int a24_side_begin(void* stream, void** side)
+{
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    SideStream* e = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(side_mu);
+        for (int i = 0; i < side_used && !e; i++)
+            if (side_table[i].owner == s)
+                e = &side_table[i];
+        if (!e && side_used < 32) {
+            SideStream n{s, nullptr, nullptr, nullptr};
+            if (hipStreamCreateWithFlags(&n.side, hipStreamNonBlocking) != hipSuccess
+                || hipEventCreateWithFlags(&n.fork, hipEventDisableTiming) != hipSuccess
+                || hipEventCreateWithFlags(&n.join, hipEventDisableTiming) != hipSuccess) {
+                (void)hipGetLastError();
+            } else {
+                side_table[side_used] = n;
+                e = &side_table[side_used++];
+            }
+        }
+    }
+    if (!e) {
+        *side = stream;
+        return 0;
+    }
+    hipError_t rc = hipEventRecord(e->fork, s);
+    if (rc == hipSuccess)
+        rc = hipStreamWaitEvent(e->side, e->fork, 0);
+    *side = e->side;
+    return static_cast<int>(rc);
+}
+
+// Everything enqueued on `side` so far happens before what is then enqueued on `stream`.
+extern "C" int a24_side_end(void* stream, void* side)
+{
+    if (side == stream)
+        return 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    std::lock_guard<std::mutex> lock(side_mu);
+    for (int i = 0; i < side_used; i++) {
+        if (side_table[i].owner == s) {
+            hipError_t rc = hipEventRecord(side_table[i].join, side_table[i].side);
+            if (rc == hipSuccess)
+                rc = hipStreamWaitEvent(s, side_table[i].join, 0);
+            return static_cast<int>(rc);
+        }
+    }
+    return static_cast<int>(hipErrorInvalidValue);
+}

@@ -7,6 +7,7 @@
 #include <mutex>
 
 #include "../../include/SpMM_API.h"
+#include "a24_format.h"
 #include "launch_plan.h"
 #include "tiled_csl_format.h"
 
@@ -18,6 +19,10 @@ int tcsl_launch_reduce(void* stream, void* C, const void* W, long rows, long vec
 int tcsl_launch_copy(void* stream, void* dst, const void* src, long bytes);
 int tcsl_launch_encode_offsets(void* stream, const void* A, int M, int K, int* offsets);
 int tcsl_launch_encode_items(void* stream, const void* A, int M, int K, const int* offsets, void* items);
+int a24_launch_spmm(void* stream, const void* packed, const void* B, void* out, int M, int N, int K, int split_k, int rb,
+                    int waves, long ldb, long ldo, long slab);
+int a24_side_begin(void* stream, void** side);
+int a24_side_end(void* stream, void* side);
 void* tcsl_event_create(void);
 void tcsl_event_destroy(void* e);
 int tcsl_event_record(void* e, void* stream);
@@ -358,4 +363,144 @@ extern "C" int SpMM_CalibrationCopy(void* stream, void* dst, const void* src, lo
     if (!dst || !src || bytes < 0 || bytes % 16 != 0)
         return tcsl_error_invalid_value();
     return tcsl_launch_copy(stream, dst, src, bytes);
+}
+
+// ---------------------------------------------------------------------------------------------
+// 2:4 part on the sparse matrix cores + Tiled-CSL residual
+
+extern "C" int HeteroSparse_Decompose(const uint16_t* A_h, uint16_t* A1_h, uint16_t* A2_h, long Length)
+{
+    if (!A_h || !A1_h || !A2_h)
+        return a24::kErrNullPointer;
+    if (Length < 0 || Length % 4 != 0)  // the reference asserts this (kernel_benchmark/spmm_decompose.h:17)
+        return a24::kErrBadShape;
+    a24::decompose(A_h, A1_h, A2_h, Length);
+    return 0;
+}
+
+extern "C" long HeteroSparse_PackedBytes(int M, int K)
+{
+    if (M <= 0 || K <= 0 || M % a24::kRows != 0 || K % a24::kUnitCols != 0)
+        return a24::kErrBadShape;
+    return a24::bytes(M, K);
+}
+
+extern "C" int HeteroSparse_PackA1(const uint16_t* A1_h, int M, int K, void* Packed_h)
+{
+    return a24::pack(A1_h, M, K, static_cast<uint8_t*>(Packed_h));
+}
+
+namespace {
+
+// Launch shape of the 2:4 kernel: row blocks per workgroup, waves per workgroup, split-K.
+struct A24Plan {
+    int row_blocks, waves, split_k;
+};
+
+A24Plan a24_default_plan(int M, int N, int K)
+{
+    // From a sweep on the OPT-30B shapes: as many rows per wave as the registers hold (a wave's
+    // activation fragments are shared by its row blocks), four waves per workgroup, and split-K
+    // until about two workgroups per compute unit exist (one for N >= 32).
+    A24Plan p{N == 64 ? 4 : 8, 4, 1};
+    const long groups = M / (16 * p.row_blocks);
+    const long target = N <= 16 ? 448 : 224;
+    const int units = K / a24::kUnitCols;
+    while (groups * p.split_k < target) {
+        const int s2 = p.split_k * 2;
+        const int per = (units + s2 - 1) / s2;
+        if (per < 2 || static_cast<long>(per) * (s2 - 1) >= units)
+            break;
+        p.split_k = s2;
+    }
+    return p;
+}
+
+bool a24_shape_ok(int M, int N, int K, int split_k, int row_blocks, int waves)
+{
+    if (N != 8 && N != 16 && N != 32 && N != 64)
+        return false;
+    if (M <= 0 || K <= 0 || M % 128 != 0 || K % a24::kUnitCols != 0 || split_k < 1 || split_k > 65535)
+        return false;
+    const int units = K / a24::kUnitCols;
+    const int per_batch = (units + split_k - 1) / split_k;
+    if (static_cast<long>(per_batch) * (split_k - 1) >= units)  // the last batch would be empty
+        return false;
+    if (row_blocks < 1 || row_blocks > 8 || (row_blocks & (row_blocks - 1)) || waves < 1 || waves > 8)
+        return false;
+    if (N == 64 && (row_blocks == 8 || (row_blocks == 4 && waves == 8)))  // accumulators would not fit the registers
+        return false;
+    return true;
+}
+
+}  // namespace
+
+extern "C" int HeteroSparse_A1_Partials(void* stream, const void* Packed_A1, const void* B, void* Partials, int M, int N,
+                                        int K, int Split_K, int RowBlocks, int Waves)
+{
+    A24Plan p{RowBlocks, Waves, Split_K};
+    if (RowBlocks == 0 || Waves == 0) {
+        const A24Plan d = a24_default_plan(M > 0 ? M : 128, N, K > 0 ? K : 128);
+        p.row_blocks = d.row_blocks;
+        p.waves = d.waves;
+    }
+    if (!Packed_A1 || !B || !Partials || !a24_shape_ok(M, N, K, p.split_k, p.row_blocks, p.waves)) {
+        std::fprintf(stderr, "HeteroSparse_A1_Partials: unsupported call M=%d N=%d K=%d Split_K=%d (need M %% 128 == 0, K %% 128 == 0, N in {8,16,32,64}, no empty batch)\n",
+                     M, N, K, Split_K);
+        return tcsl_error_invalid_value();
+    }
+    return a24_launch_spmm(stream, Packed_A1, B, Partials, M, N, K, p.split_k, p.row_blocks, p.waves, K, M,
+                           static_cast<long>(M) * N);
+}
+
+extern "C" int HeteroSparse_SuggestSplitK(int M, int N, int K)
+{
+    if (!a24_shape_ok(M, N, K, 1, 1, 1))
+        return 1;
+    return a24_default_plan(M, N, K).split_k;
+}
+
+extern "C" int HeteroSparse_SpMM_API(void* stream, const void* Packed_A1, const void* Compressed_A2,
+                                     const int* TileOffsets_A2, const void* B, void* C, int M, int N, int K,
+                                     void* Reduction_Workspace, int Split_K_A1, int Split_K_A2, int Flags)
+{
+    const bool residual = Compressed_A2 != nullptr;
+    if (N != 8 && N != 16 && N != 32 && N != 64) {
+        std::printf("MM_Sparse_API Error: Unsupported N dimension %d!\n", N);  // csrc/SpMM_API.cu:192-193
+        return tcsl_error_unknown();
+    }
+    const A24Plan d = a24_shape_ok(M, N, K, Split_K_A1, 1, 1) ? a24_default_plan(M, N, K) : A24Plan{1, 1, 1};
+    if (!Packed_A1 || !B || !C || (residual && !TileOffsets_A2) || !a24_shape_ok(M, N, K, Split_K_A1, d.row_blocks, d.waves)
+        || (residual && (Split_K_A2 < 1 || Split_K_A2 > 65535)) || ((residual || Split_K_A1 > 1) && !Reduction_Workspace)
+        || (Flags & ~HETERO_FLAG_TWO_STREAMS)) {
+        std::fprintf(stderr, "HeteroSparse_SpMM_API: unsupported call M=%d N=%d K=%d Split_K=%d/%d (need M %% 128 == 0, K %% 128 == 0, no empty batch, non-null pointers)\n",
+                     M, N, K, Split_K_A1, Split_K_A2);
+        return tcsl_error_invalid_value();
+    }
+    const long mn = static_cast<long>(M) * N;
+    if (!residual && Split_K_A1 == 1)  // the 2:4 kernel writes C itself
+        return a24_launch_spmm(stream, Packed_A1, B, C, M, N, K, 1, d.row_blocks, d.waves, K, M, mn);
+    int rc = 0;
+    int slabs = Split_K_A1;
+    if (residual) {
+        // On request the residual's kernel goes to a second stream, beside the 2:4 kernel.  Measured
+        // slower than one stream (two event waits cost more than the overlap gains), hence optional.
+        void* side = stream;
+        if ((Flags & HETERO_FLAG_TWO_STREAMS) && (rc = a24_side_begin(stream, &side)) != 0)
+            return rc;
+        rc = launch_main(side, Compressed_A2, TileOffsets_A2, B, static_cast<uint16_t*>(Reduction_Workspace) + slabs * mn, M,
+                         N, K, Split_K_A2, CallOptions{}, K, M, false, nullptr, 0, nullptr);
+        if (rc != 0)
+            return rc;
+        slabs += Split_K_A2;
+        rc = a24_launch_spmm(stream, Packed_A1, B, Reduction_Workspace, M, N, K, Split_K_A1, d.row_blocks, d.waves, K, M, mn);
+        if (rc != 0)
+            return rc;
+        if ((rc = a24_side_end(stream, side)) != 0)
+            return rc;
+    } else if ((rc = a24_launch_spmm(stream, Packed_A1, B, Reduction_Workspace, M, N, K, Split_K_A1, d.row_blocks, d.waves, K,
+                                     M, mn)) != 0) {
+        return rc;
+    }
+    return tcsl_launch_reduce(stream, C, Reduction_Workspace, mn, 1, mn, slabs, 0);
 }

@@ -9,6 +9,9 @@ Reference interfaces mirrored (paths relative to the reference checkout):
   SpMM_SplitK_API         third_party/ft.patch:2833-2843, csrc/SpMM_API.cu:79-208
   GenSparseMatrixBinFile  csrc/SpMM_API.cu:1565-1620,
                           end2end_inference/ft_tools/huggingface_opt_convert_Phase2.py:36-59
+  decompose               kernel_benchmark/spmm_decompose.h:12-51  (HeteroSparse_Decompose)
+  2:4 part + residual     kernel_benchmark/spmm_test.cu:285-330,462-560, csrc/SpMM_API.cu:1127-1553
+                          (HeteroSparse_PackA1, HeteroSparse_SpMM_API)
 """
 import ctypes
 import os
@@ -47,6 +50,12 @@ EXPORTED_SYMBOLS = (
     "SpMM_EventDestroy",
     "SpMM_EventRecord",
     "SpMM_EventElapsedMs",
+    "HeteroSparse_Decompose",
+    "HeteroSparse_PackedBytes",
+    "HeteroSparse_PackA1",
+    "HeteroSparse_SpMM_API",
+    "HeteroSparse_SuggestSplitK",
+    "HeteroSparse_A1_Partials",
 )
 
 
@@ -141,6 +150,18 @@ def load_library():
     lib.SpMM_EventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
     lib.SpMM_EventElapsedMs.restype = ctypes.c_float
     lib.SpMM_EventElapsedMs.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+    lib.HeteroSparse_Decompose.restype = ctypes.c_int
+    lib.HeteroSparse_Decompose.argtypes = [_u16p, _u16p, _u16p, ctypes.c_long]
+    lib.HeteroSparse_PackedBytes.restype = ctypes.c_long
+    lib.HeteroSparse_PackedBytes.argtypes = [ctypes.c_int, ctypes.c_int]
+    lib.HeteroSparse_PackA1.restype = ctypes.c_int
+    lib.HeteroSparse_PackA1.argtypes = [_u16p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    lib.HeteroSparse_SpMM_API.restype = ctypes.c_int
+    lib.HeteroSparse_SpMM_API.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int] * 3 + [ctypes.c_void_p] + [ctypes.c_int] * 3
+    lib.HeteroSparse_SuggestSplitK.restype = ctypes.c_int
+    lib.HeteroSparse_SuggestSplitK.argtypes = [ctypes.c_int] * 3
+    lib.HeteroSparse_A1_Partials.restype = ctypes.c_int
+    lib.HeteroSparse_A1_Partials.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 6
     _lib = lib
     return lib
 
@@ -326,3 +347,70 @@ def synth_activations(N, K, seed=0):
     B = np.empty((N, K), dtype=np.uint16)
     load_library().SpMM_SynthActivations(B.ctypes.data_as(_u16p), N * K, seed)
     return B.view(np.float16)
+
+
+# ---------------------------------------------------------------------------------------------
+# 2:4 part on the sparse matrix cores + Tiled-CSL residual
+
+
+HETERO_FLAG_TWO_STREAMS = 1
+
+
+def HeteroSparse_Decompose(A_h):
+    """(A1, A2) of a row-major fp16 matrix: at most two kept values per group of four in A1, the
+    rest in A2 (kernel_benchmark/spmm_decompose.h:12-51, bit for bit)."""
+    a = _bits(A_h)
+    A1 = np.empty(a.shape, dtype=np.uint16)
+    A2 = np.empty(a.shape, dtype=np.uint16)
+    rc = load_library().HeteroSparse_Decompose(a.ctypes.data_as(_u16p), A1.ctypes.data_as(_u16p),
+                                               A2.ctypes.data_as(_u16p), a.size)
+    if rc != 0:
+        raise SpMMError("HeteroSparse_Decompose", rc)
+    return A1.view(np.float16), A2.view(np.float16)
+
+
+def HeteroSparse_PackA1(A1_h, M=None, K=None):
+    """Records of the 2:4 part in sparse-MFMA operand order -> uint8[(M/16)*(K/128)*2304]."""
+    a = _bits(A1_h)
+    if M is None or K is None:
+        M, K = a.shape
+    lib = load_library()
+    size = lib.HeteroSparse_PackedBytes(M, K)
+    if size < 0:
+        raise SpMMError("HeteroSparse_PackedBytes", int(size))
+    packed = np.empty(size, dtype=np.uint8)
+    rc = lib.HeteroSparse_PackA1(a.ctypes.data_as(_u16p), M, K, packed.ctypes.data_as(ctypes.c_void_p))
+    if rc != 0:
+        raise SpMMError("HeteroSparse_PackA1", rc)
+    return packed
+
+
+def HeteroSparse_SuggestSplitK(M_Global, N_Global, K_Global):
+    return load_library().HeteroSparse_SuggestSplitK(M_Global, N_Global, K_Global)
+
+
+def HeteroSparse_SpMM_API(stream, Packed_A1, Compressed_A2, TileOffsets_A2, B, C, M_Global, N_Global, K_Global,
+                          Reduction_Workspace, Split_K_A1, Split_K_A2, Flags=0):
+    """Enqueue C = A1*B + A2*B (A1 as 2:4 records, A2 as Tiled-CSL or None) on `stream`."""
+    lib = load_library()
+    if stream is not None and not isinstance(stream, int):
+        stream = stream.cuda_stream
+    rc = lib.HeteroSparse_SpMM_API(ctypes.c_void_p(stream) if stream else None, _ptr(Packed_A1), _ptr(Compressed_A2),
+                                   _ptr(TileOffsets_A2), _ptr(B), _ptr(C), M_Global, N_Global, K_Global,
+                                   _ptr(Reduction_Workspace), Split_K_A1, Split_K_A2, Flags)
+    if rc != 0:
+        raise SpMMError("HeteroSparse_SpMM_API", rc, lib.SpMM_GetErrorString(rc).decode())
+    return rc
+
+
+def HeteroSparse_A1_Partials(stream, Packed_A1, B, Partials, M_Global, N_Global, K_Global, Split_K, RowBlocks=0,
+                             Waves=0):
+    """The 2:4 kernel alone, with a caller-chosen launch shape (0, 0 = the library's)."""
+    lib = load_library()
+    if stream is not None and not isinstance(stream, int):
+        stream = stream.cuda_stream
+    rc = lib.HeteroSparse_A1_Partials(ctypes.c_void_p(stream) if stream else None, _ptr(Packed_A1), _ptr(B),
+                                      _ptr(Partials), M_Global, N_Global, K_Global, Split_K, RowBlocks, Waves)
+    if rc != 0:
+        raise SpMMError("HeteroSparse_A1_Partials", rc, lib.SpMM_GetErrorString(rc).decode())
+    return rc

@@ -240,6 +240,70 @@ SPMM_EXPORT void SpMM_SynthActivations(uint16_t* B_h, long count, uint64_t seed)
  */
 SPMM_EXPORT int SpMM_CalibrationCopy(void* stream, void* dst, const void* src, long bytes);
 
+/*
+ * ---- 2:4 part on the sparse matrix cores + Tiled-CSL residual ------------------------------
+ * This checkout's own line of work: a weight is split into A1, with at most two kept values in
+ * every group of four along K (the shape sparse matrix cores take), and the residual A2, which
+ * stays in Tiled-CSL; C = A1*B + A2*B.  The reference builds A1's device form for NVIDIA's mma.sp
+ * (csrc/SpMM_API.cu:1127-1553) and passes it through two extra operands of SpMM_SplitK_API
+ * (build/SpMM_API.cuh:40-52), with A2 going to a second kernel on another stream
+ * (kernel_benchmark/spmm_test.cu:285-330,462-560).  Here A1 is stored as records in the operand
+ * order of gfx950's v_smfmac_f32_16x16x32_f16 (16 rows x 128 columns, 2304 bytes: 2048 bytes of
+ * fp16 values, 256 bytes of 2-bit positions; 1.125 bytes per dense element at any sparsity).
+ */
+
+/*
+ * Stands in for  void decompose(half* A, half* A1, half* A2, int length)
+ * (kernel_benchmark/spmm_decompose.h:12-51), bit for bit: in each group of four consecutive
+ * elements the first two that compare unequal to zero (NaN counts, -0 does not) go to A1, the
+ * others to A2; everything else is +0.  Host memory, fp16 bit patterns, Length % 4 == 0.
+ * Returns 0, -1 (bad length) or -3 (null pointer) where the reference asserts; prints nothing.
+ */
+SPMM_EXPORT int HeteroSparse_Decompose(const uint16_t* A_h, uint16_t* A1_h, uint16_t* A2_h, long Length);
+
+/*
+ * Stand in for InitSparseMatrixA1_Vec_Sparse_Load and inspect_metadata (csrc/SpMM_API.cu:1127-1553),
+ * which produce mma.sp's value and metadata arrays; the bytes differ by design (other hardware).
+ * HeteroSparse_PackedBytes: size of the records of an M x K matrix (M % 16 == 0, K % 128 == 0), or -1.
+ * HeteroSparse_PackA1: fills Packed_h (host memory of that size) from row-major A1_h.  Returns 0,
+ * -1 bad shape, -3 null pointer, -6 if some group of four holds more than two kept values.
+ */
+SPMM_EXPORT long HeteroSparse_PackedBytes(int M, int K);
+SPMM_EXPORT int HeteroSparse_PackA1(const uint16_t* A1_h, int M, int K, void* Packed_h);
+
+/*
+ * C = A1*B + A2*B on the GPU; the counterpart of this checkout's 13-argument SpMM_SplitK_API call
+ * followed by its residual kernel and reduction (kernel_benchmark/spmm_test.cu:462-560).
+ * Packed_A1: device copy of the records; Compressed_A2 / TileOffsets_A2: device Tiled-CSL of the
+ * residual (InitSparseMatrixA_API on A2), or both NULL when there is none.  B[N][K], C[N][M] as
+ * for SpMM_SplitK_API.  The 2:4 kernel writes Split_K_A1 slabs of fp16 partial sums, the
+ * Tiled-CSL kernel Split_K_A2 more, and one reduction adds them up in fp32: Reduction_Workspace
+ * must hold (Split_K_A1 + Split_K_A2)*M*N fp16 values.  With no residual and Split_K_A1 == 1 the
+ * workspace is not touched.  HeteroSparse_SuggestSplitK gives a Split_K_A1 that fills the chip.
+ * The kernels run one after the other on `stream`.  Flags = HETERO_FLAG_TWO_STREAMS sends the
+ * residual's kernel to a second stream that the library keeps per caller stream (default priority,
+ * made on first use; the reference gives the two parts their own streams,
+ * kernel_benchmark/spmm_test.cu:459-461), ordered after what `stream` held before the call, with
+ * the reduction on `stream` waiting for both; on an MI355X that measured slower than one stream.
+ * Returns a hipError_t value: hipErrorUnknown for N outside {8, 16, 32, 64};
+ * hipErrorInvalidValue for M % 128, K % 128, a split that leaves a batch of 128-column units
+ * empty, or a missing pointer.  Only enqueues work on `stream`.  Thread safe.
+ */
+#define HETERO_FLAG_TWO_STREAMS 1
+SPMM_EXPORT int HeteroSparse_SpMM_API(void* stream, const void* Packed_A1, const void* Compressed_A2,
+                                      const int* TileOffsets_A2, const void* B, void* C, int M_Global, int N_Global,
+                                      int K_Global, void* Reduction_Workspace, int Split_K_A1, int Split_K_A2, int Flags);
+SPMM_EXPORT int HeteroSparse_SuggestSplitK(int M_Global, int N_Global, int K_Global);
+
+/*
+ * The 2:4 kernel alone: batch b of ceil((K/128)/Split_K) units writes fp16 A1*B partial sums to
+ * Partials[b*M*N ..).  RowBlocks (16-row blocks per workgroup: 1, 2, 4, 8) and Waves (waves per
+ * workgroup that split the batch: 1, 2, 4, 8) choose the launch shape; 0, 0 = the library's
+ * choice.  hipErrorInvalidValue for shapes the kernel table does not hold.  For tuning and tests.
+ */
+SPMM_EXPORT int HeteroSparse_A1_Partials(void* stream, const void* Packed_A1, const void* B, void* Partials, int M_Global,
+                                         int N_Global, int K_Global, int Split_K, int RowBlocks, int Waves);
+
 #ifdef __cplusplus
 }
 #endif

@@ -48,6 +48,9 @@ def _load():
     lib.oracle_spmm_splitk.restype = ctypes.c_int
     lib.oracle_spmm_splitk.argtypes = [_u32p, _i32p, _u16p, _u16p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u16p,
                                        ctypes.c_int]
+    lib.oracle_decompose.argtypes = [_u16p, _u16p, _u16p, ctypes.c_long]
+    lib.oracle_a24_unpack.restype = ctypes.c_int
+    lib.oracle_a24_unpack.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, _u16p]
     return lib
 
 
@@ -151,6 +154,26 @@ def spmm_splitk(items, offsets, B, M, N, K, split_k):
     return C.view(np.float16), W.view(np.float16)
 
 
+def decompose(A):
+    """2:4 part and residual of a row-major fp16 matrix (kernel_benchmark/spmm_decompose.h:12-51)."""
+    a = _bits(A)
+    A1 = np.empty(a.shape, dtype=np.uint16)
+    A2 = np.empty(a.shape, dtype=np.uint16)
+    lib().oracle_decompose(a.ctypes.data_as(_u16p), A1.ctypes.data_as(_u16p), A2.ctypes.data_as(_u16p), a.size)
+    return A1.view(np.float16), A2.view(np.float16)
+
+
+def a24_unpack(packed, M, K):
+    """Dense fp16 M x K matrix held by 2:4 records (16 rows x 128 columns, 2304 bytes each)."""
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    assert packed.size == (M // 16) * (K // 128) * 2304, packed.size
+    out = np.empty((M, K), dtype=np.uint16)
+    rc = lib().oracle_a24_unpack(packed.ctypes.data_as(ctypes.c_void_p), M, K, out.ctypes.data_as(_u16p))
+    if rc:
+        raise ValueError("2:4 records with equal or descending positions inside a group")
+    return out.view(np.float16)
+
+
 # ----------------------------------------------------------------------------
 # the reference's own encoder, where oracle/_ref was built
 
@@ -183,3 +206,16 @@ def ref_encode(A, reorder=True):
     it = _take(items, int(o[-1]) * 4, np.uint32, _ref.ref_free)
     _ref.ref_free(offs)
     return it, o
+
+
+def ref_decompose(A):
+    """The reference's own decompose() (kernel_benchmark/spmm_decompose.h:12-51); prints its statistics."""
+    global _ref
+    if _ref is None:
+        ref_encode(np.zeros((128, 64), dtype=np.float16))  # loads the library
+    _ref.ref_decompose.argtypes = [_u16p, _u16p, _u16p, ctypes.c_int]
+    a = _bits(A).copy()
+    A1 = np.empty(a.shape, dtype=np.uint16)
+    A2 = np.empty(a.shape, dtype=np.uint16)
+    _ref.ref_decompose(a.ctypes.data_as(_u16p), A1.ctypes.data_as(_u16p), A2.ctypes.data_as(_u16p), a.size)
+    return A1.view(np.float16), A2.view(np.float16)

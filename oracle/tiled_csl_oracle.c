@@ -27,6 +27,14 @@
  *   oracle_spmm_splitk   - composition of the above; sum of slabs equals the
  *                          full product.
  *   half conversions     - exhaustive comparison with numpy float16.
+ *   oracle_decompose     - bit-compared with the reference's own decompose()
+ *                          compiled from kernel_benchmark/spmm_decompose.h:12-51
+ *                          (oracle/_ref); A1 + A2 == A with disjoint supports; at
+ *                          most two kept values per group of four in A1; hand cases.
+ *   oracle_a24_unpack    - reader of this build's 2:4 record layout (the reference's
+ *                          own on-device form, csrc/SpMM_API.cu:1127-1553, is made for
+ *                          NVIDIA's mma.sp and has no meaning here); pinned by
+ *                          hand-built records and by unpack(pack(A1)) == A1.
  */
 #include <stdint.h>
 #include <stdlib.h>
@@ -435,5 +443,73 @@ int oracle_spmm_splitk(const uint32_t *items, const int *offsets, const uint16_t
         oracle_reduce(C, workspace, MN, Split_K);
     free(A);
     free(acc);
+    return 0;
+}
+
+
+/* ------------------------------------------------- 2:4 + residual split -- */
+
+/*
+ * kernel_benchmark/spmm_decompose.h:12-51.  The flat array is cut into groups of
+ * four consecutive elements; in each group the first two values that compare
+ * unequal to zero as floats (so NaN counts, -0 does not) go to A1 at their own
+ * positions, every further one goes to A2.  Both outputs are zero-filled first.
+ */
+void oracle_decompose(const uint16_t *A, uint16_t *A1, uint16_t *A2, long length)
+{
+    memset(A1, 0, sizeof(uint16_t) * (size_t)length);
+    memset(A2, 0, sizeof(uint16_t) * (size_t)length);
+    for (long i = 0; i + 3 < length; i += 4) {
+        int taken = 0;
+        for (int e = 0; e < 4; e++) {
+            if (oracle_half_to_float(A[i + e]) != 0.0f) {
+                if (taken < 2)
+                    A1[i + e] = A[i + e];
+                else
+                    A2[i + e] = A[i + e];
+                taken++;
+            }
+        }
+    }
+}
+
+/*
+ * Reader of the 2:4 records that the sparse-MFMA kernel streams.  One record covers
+ * 16 rows x 128 columns and is 2304 bytes: for lane L in 0..63 (row L % 16, column
+ * group g = L / 16), step s in 0..3 and slot j in 0..3, the fp16 value at byte
+ * (s / 2) * 1024 + L * 16 + ((s % 2) * 4 + j) * 2 belongs to column
+ * s * 32 + g * 8 + (j / 2) * 4 + q of the record, where q is the 2-bit field at bit
+ * 8 * s + 2 * j of the 32-bit word at byte 2048 + L * 4.  Records are ordered by
+ * 16-row block, then by 128-column unit.  Returns 0, or -1 if two slots of one group
+ * of four name the same column or come in descending order.
+ */
+int oracle_a24_unpack(const uint8_t *packed, int M, int K, uint16_t *A_out)
+{
+    const int units = K / 128;
+    memset(A_out, 0, sizeof(uint16_t) * (size_t)M * (size_t)K);
+    for (int rb = 0; rb < M / 16; rb++) {
+        for (int u = 0; u < units; u++) {
+            const uint8_t *rec = packed + ((size_t)rb * units + u) * 2304;
+            for (int L = 0; L < 64; L++) {
+                uint32_t word;
+                memcpy(&word, rec + 2048 + L * 4, 4);
+                for (int s = 0; s < 4; s++) {
+                    for (int j = 0; j < 4; j++) {
+                        uint16_t v;
+                        memcpy(&v, rec + (s / 2) * 1024 + L * 16 + ((s % 2) * 4 + j) * 2, 2);
+                        int q = (int)((word >> (8 * s + 2 * j)) & 3u);
+                        if (j % 2 == 1) {
+                            int q_prev = (int)((word >> (8 * s + 2 * (j - 1))) & 3u);
+                            if (q_prev >= q)
+                                return -1;
+                        }
+                        size_t row = (size_t)rb * 16 + (size_t)(L % 16);
+                        size_t col = (size_t)u * 128 + (size_t)(s * 32 + (L / 16) * 8 + (j / 2) * 4 + q);
+                        A_out[row * (size_t)K + col] = v;
+                    }
+                }
+            }
+        }
+    }
     return 0;
 }

@@ -1,0 +1,148 @@
+"""CPU tests of the 2:4 + residual split and of the 2:4 record packer.
+
+decompose() is pinned three ways: the oracle against the reference's own function compiled
+from kernel_benchmark/spmm_decompose.h:12-51 (oracle/_ref, where that build ran), hand-made
+groups whose answer is read off the reference's loop, and the properties the split must have.
+The product's HeteroSparse_Decompose is then compared with the oracle bit for bit.
+The record layout is this build's own (the reference's is made for NVIDIA's mma.sp); the
+oracle's reader is pinned by records built by hand here, byte by byte, and the packer by
+unpack(pack(A1)) == A1.
+"""
+import numpy as np
+import pytest
+
+H = np.float16
+
+
+def _rand_sparse(rng, M, K, keep):
+    A = (rng.standard_normal((M, K)) * 0.02).astype(H)
+    A[rng.random((M, K)) >= keep] = 0
+    return A
+
+
+def test_oracle_decompose_hand_cases(oracle):
+    nan = np.array([0x7E00], dtype=np.uint16).view(H)[0]
+    negzero = np.array([0x8000], dtype=np.uint16).view(H)[0]
+    A = np.array([
+        [1, 2, 3, 4],          # first two stay, last two go to the residual
+        [0, 5, 0, 6],          # already 2:4
+        [7, 0, 8, 9],          # third kept value (9) is the residual
+        [0, 0, 0, 0],
+        [negzero, 1, 2, 3],    # -0 compares equal to zero: 1, 2 stay, 3 goes
+        [nan, 1, 2, 0],        # NaN compares unequal: NaN, 1 stay, 2 goes
+    ], dtype=H)
+    A1, A2 = oracle.decompose(A)
+    e1 = np.array([[1, 2, 0, 0], [0, 5, 0, 6], [7, 0, 8, 0], [0, 0, 0, 0], [0, 1, 2, 0], [nan, 1, 0, 0]], dtype=H)
+    e2 = np.array([[0, 0, 3, 4], [0, 0, 0, 0], [0, 0, 0, 9], [0, 0, 0, 0], [0, 0, 0, 3], [0, 0, 2, 0]], dtype=H)
+    assert np.array_equal(A1.view(np.uint16), e1.view(np.uint16))
+    assert np.array_equal(A2.view(np.uint16), e2.view(np.uint16))
+
+
+@pytest.mark.parametrize("keep", [0.1, 0.3, 0.5, 0.9])
+def test_oracle_decompose_properties(oracle, keep):
+    rng = np.random.default_rng(int(keep * 100))
+    A = _rand_sparse(rng, 64, 256, keep)
+    A1, A2 = oracle.decompose(A)
+    nz, nz1, nz2 = A != 0, A1 != 0, A2 != 0
+    assert not (nz1 & nz2).any()
+    assert np.array_equal(np.where(nz1, A1, A2).view(np.uint16), np.where(nz, A, H(0)).view(np.uint16))
+    g = nz.reshape(-1, 4)
+    assert np.array_equal(nz1.reshape(-1, 4).sum(1), np.minimum(g.sum(1), 2))
+    # the residual takes the LAST kept values of a group: rank of a kept value within its group >= 2
+    rank = np.cumsum(g, axis=1) - 1
+    assert np.array_equal(nz2.reshape(-1, 4), g & (rank >= 2))
+
+
+def test_oracle_decompose_matches_reference_build(oracle):
+    if not oracle.have_ref():
+        pytest.skip("oracle/_ref not built (no reference checkout on this machine)")
+    rng = np.random.default_rng(11)
+    for keep in (0.2, 0.5, 0.8):
+        A = _rand_sparse(rng, 128, 512, keep)
+        A.view(np.uint16)[0, :8] = [0x8000, 0x7E00, 0x0001, 0x3C00, 0xFC00, 0x8001, 0, 0x7C00]
+        o1, o2 = oracle.decompose(A)
+        r1, r2 = oracle.ref_decompose(A)
+        assert np.array_equal(o1.view(np.uint16), r1.view(np.uint16))
+        assert np.array_equal(o2.view(np.uint16), r2.view(np.uint16))
+
+
+@pytest.mark.parametrize("keep", [0.0, 0.2, 0.5, 1.0])
+def test_product_decompose_equals_oracle(spmm, oracle, keep):
+    rng = np.random.default_rng(7)
+    A = _rand_sparse(rng, 128, 384, keep)
+    A.view(np.uint16)[1, :4] = [0x8000, 0x7E00, 0x0001, 0x3C00]
+    p1, p2 = spmm.HeteroSparse_Decompose(A)
+    o1, o2 = oracle.decompose(A)
+    assert np.array_equal(p1.view(np.uint16), o1.view(np.uint16))
+    assert np.array_equal(p2.view(np.uint16), o2.view(np.uint16))
+
+
+def test_decompose_rejects_bad_length(spmm):
+    with pytest.raises(spmm.SpMMError):
+        spmm.HeteroSparse_Decompose(np.zeros(6, dtype=H))
+
+
+def test_oracle_unpack_reads_a_hand_built_record(oracle):
+    """One 16 x 128 record written byte by byte from the layout's definition."""
+    M, K = 16, 128
+    rec = np.zeros(2304, dtype=np.uint8)
+    words = np.zeros(64, dtype=np.uint32)
+    for L in range(64):  # every group of four: positions (0, 1), zero values
+        for s in range(4):
+            for j in range(4):
+                words[L] |= np.uint32((j % 2)) << np.uint32(8 * s + 2 * j)
+    expect = np.zeros((M, K), dtype=H)
+
+    def put(L, s, j, q_pair, value):
+        # slot j of lane L in step s holds `value` at position q_pair[j % 2]; the pair is ascending
+        for t in range(2):
+            jj = (j // 2) * 2 + t
+            shift = 8 * s + 2 * jj
+            words[L] = (int(words[L]) & ~(3 << shift)) | (q_pair[t] << shift)
+        off = (s // 2) * 1024 + L * 16 + ((s % 2) * 4 + j) * 2
+        rec[off:off + 2] = np.array([value], dtype=H).view(np.uint8)
+        expect[L % 16, s * 32 + (L // 16) * 8 + (j // 2) * 4 + q_pair[j % 2]] = value
+
+    put(0, 0, 0, (0, 1), 1.5)      # row 0, column 0
+    put(0, 0, 3, (1, 3), -2.0)     # row 0, second group of the lane: column 4 + 3
+    put(17, 2, 1, (2, 3), 3.0)     # row 1, column 2*32 + 1*8 + 3
+    put(63, 3, 2, (1, 2), 0.25)    # row 15, column 3*32 + 3*8 + 4 + 1
+    rec[2048:] = words.view(np.uint8)
+    got = oracle.a24_unpack(rec, M, K)
+    assert np.array_equal(got.view(np.uint16), expect.view(np.uint16))
+    assert got[0, 0] == H(1.5) and got[0, 7] == H(-2.0) and got[1, 75] == H(3.0) and got[15, 125] == H(0.25)
+    words[5] = 0  # positions (0, 0) in every pair: not a valid record
+    rec[2048:] = words.view(np.uint8)
+    with pytest.raises(ValueError):
+        oracle.a24_unpack(rec, M, K)
+
+
+@pytest.mark.parametrize("M,K,keep", [(16, 128, 0.5), (128, 256, 0.2), (256, 1024, 0.8), (128, 128, 0.0)])
+def test_pack_round_trip(spmm, oracle, M, K, keep):
+    rng = np.random.default_rng(M + K)
+    A1, _ = oracle.decompose(_rand_sparse(rng, M, K, keep))
+    packed = spmm.HeteroSparse_PackA1(A1)
+    assert packed.size == (M // 16) * (K // 128) * 2304
+    back = oracle.a24_unpack(packed, M, K)  # also checks ascending positions in every group
+    assert np.array_equal(back.view(np.uint16), A1.view(np.uint16))
+
+
+def test_pack_rejects_three_of_four_and_bad_shapes(spmm):
+    A = np.zeros((16, 128), dtype=H)
+    A[3, 8:11] = 1
+    with pytest.raises(spmm.SpMMError) as e:
+        spmm.HeteroSparse_PackA1(A)
+    assert e.value.code == -6
+    with pytest.raises(spmm.SpMMError):
+        spmm.HeteroSparse_PackA1(np.zeros((16, 64), dtype=H))
+    with pytest.raises(spmm.SpMMError):
+        spmm.HeteroSparse_PackA1(np.zeros((8, 128), dtype=H))
+
+
+def test_suggested_split_leaves_no_batch_empty(spmm):
+    for M, K in [(28672, 7168), (7168, 28672), (7168, 7168), (9216, 36864), (128, 128), (256, 384)]:
+        for N in (8, 16, 32, 64):
+            s = spmm.HeteroSparse_SuggestSplitK(M, N, K)
+            units = K // 128
+            per = -(-units // s)
+            assert s >= 1 and per * (s - 1) < units
