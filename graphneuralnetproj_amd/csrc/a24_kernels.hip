@@ -184,6 +184,178 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_kernel(const uint8_t* __res
     }
 }
 
+// The other work split, for wide token counts: the W waves of a workgroup own RB row blocks each
+// (16 * RB * W rows per workgroup) and walk the batch's units together.  The unit's activation
+// tile (n_tokens x 128 fp16) is fetched once per workgroup with full-line loads, kept in LDS
+// (two buffers, rows padded to 272 bytes so that the sixteen lanes of a quarter wave read sixteen
+// different bank groups) and read back by every wave in operand order: a wave's fragments come
+// from LDS instead of the L2, and no sum across waves is needed at the end.
+constexpr int kRowBytes = 272;
+
+template<int NT, int RB, int W>
+__global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8_t* __restrict__ packed,
+                                                                     const _Float16* __restrict__ B,
+                                                                     _Float16* __restrict__ out, int units,
+                                                                     int units_per_batch, long ldb, long ldo, long slab,
+                                                                     int n_tokens)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char tile[];  // [2][NT * 16][kRowBytes]
+    constexpr int kBuf = NT * 16 * kRowBytes;
+    constexpr int kThreads = W * kWave;
+    constexpr int CH = (NT * 256 + kThreads - 1) / kThreads;  // 16-byte chunks of a tile per thread
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    const int batch = blockIdx.y;
+    const int u0 = batch * units_per_batch;
+    const int u1 = min(units, u0 + units_per_batch);
+    const int block0 = (blockIdx.x * W + wave) * RB;
+
+    const uint8_t* rec[RB];
+#pragma unroll
+    for (int r = 0; r < RB; r++)
+        rec[r] = packed + ((size_t)(block0 + r) * units) * kRecordBytes;
+    // this thread's chunks of the activation tile: token c / 16, columns (c % 16) * 8 .. + 8
+    const _Float16* src[CH];
+    int dst[CH];
+    bool mine[CH];
+#pragma unroll
+    for (int i = 0; i < CH; i++) {
+        const int c = tid + i * kThreads;
+        mine[i] = c < n_tokens * 16;
+        const int n = mine[i] ? c >> 4 : 0;
+        src[i] = B + (size_t)n * ldb + (c & 15) * 8;
+        dst[i] = n * kRowBytes + (c & 15) * 16;
+    }
+    // where this lane's fragments sit in a buffer
+    int frag[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        int n = t * 16 + (lane & 15);
+        n = n < n_tokens ? n : n_tokens - 1;
+        frag[t] = n * kRowBytes + (lane >> 4) * 16;
+    }
+
+    float4v acc[RB][NT];
+#pragma unroll
+    for (int r = 0; r < RB; r++)
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+            acc[r][t] = float4v{0.f, 0.f, 0.f, 0.f};
+
+    u32x4 stage[CH];
+    auto fetch_b = [&](int u) {
+#pragma unroll
+        for (int i = 0; i < CH; i++)
+            if (mine[i])
+                stage[i] = *reinterpret_cast<const u32x4*>(src[i] + (size_t)u * 128);
+    };
+    auto store_b = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < CH; i++)
+            if (mine[i])
+                *reinterpret_cast<u32x4*>(tile + buf * kBuf + dst[i]) = stage[i];
+    };
+    auto multiply_from = [&](const AFrag(&a)[RB], int buf) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            half8 f[4];
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+                f[s] = *reinterpret_cast<const half8*>(tile + buf * kBuf + frag[t] + s * 64);
+#pragma unroll
+            for (int r = 0; r < RB; r++) {
+                acc[r][t] = __builtin_amdgcn_smfmac_f32_16x16x32_f16(step_values(a[r], 0), f[0], acc[r][t], (int)a[r].idx, 0, 0);
+                acc[r][t] = __builtin_amdgcn_smfmac_f32_16x16x32_f16(step_values(a[r], 1), f[1], acc[r][t], (int)a[r].idx, 0, 1);
+                acc[r][t] = __builtin_amdgcn_smfmac_f32_16x16x32_f16(step_values(a[r], 2), f[2], acc[r][t], (int)a[r].idx, 0, 2);
+                acc[r][t] = __builtin_amdgcn_smfmac_f32_16x16x32_f16(step_values(a[r], 3), f[3], acc[r][t], (int)a[r].idx, 0, 3);
+            }
+        }
+    };
+
+    AFrag a0[RB], a1[RB];
+    int u = u0;  // every wave of the workgroup walks the same units: the barriers below are uniform
+    if (u < u1) {
+        fetch_b(u);
+#pragma unroll
+        for (int r = 0; r < RB; r++)
+            a0[r] = load_a(rec[r] + (size_t)u * kRecordBytes, lane);
+        store_b(0);
+        __syncthreads();
+        while (true) {
+            // even unit: records in a0, tile in buffer 0
+            bool more = u + 1 < u1;
+            if (more) {
+                fetch_b(u + 1);
+#pragma unroll
+                for (int r = 0; r < RB; r++)
+                    a1[r] = load_a(rec[r] + (size_t)(u + 1) * kRecordBytes, lane);
+            }
+            multiply_from(a0, 0);
+            if (!more)
+                break;
+            store_b(1);  // buffer 1 was last read before the previous barrier
+            __syncthreads();
+            ++u;
+            // odd unit: records in a1, tile in buffer 1
+            more = u + 1 < u1;
+            if (more) {
+                fetch_b(u + 1);
+#pragma unroll
+                for (int r = 0; r < RB; r++)
+                    a0[r] = load_a(rec[r] + (size_t)(u + 1) * kRecordBytes, lane);
+            }
+            multiply_from(a1, 1);
+            if (!more)
+                break;
+            store_b(0);
+            __syncthreads();
+            ++u;
+        }
+    }
+
+    _Float16* dstc = out + (size_t)batch * slab;
+#pragma unroll
+    for (int r = 0; r < RB; r++) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int n = t * 16 + (lane & 15);
+            if (n < n_tokens) {
+                const float4v s = acc[r][t];
+                half4 h = {static_cast<_Float16>(s[0]), static_cast<_Float16>(s[1]), static_cast<_Float16>(s[2]),
+                           static_cast<_Float16>(s[3])};
+                *reinterpret_cast<half4*>(dstc + (size_t)n * ldo + (block0 + r) * 16 + (lane >> 4) * 4) = h;
+            }
+        }
+    }
+}
+
+template<int NT, int RB, int W>
+int launch_shared_b(hipStream_t stream, const void* packed, const void* B, void* out, int M, int N, int K, int split_k,
+                    long ldb, long ldo, long slab)
+{
+    const int units = K / 128;
+    const int per_batch = (units + split_k - 1) / split_k;
+    if (M % (16 * RB * W) != 0)
+        return static_cast<int>(hipErrorInvalidValue);
+    hipLaunchKernelGGL((a24_spmm_shared_b_kernel<NT, RB, W>), dim3(M / (16 * RB * W), split_k), dim3(W * kWave),
+                       2 * NT * 16 * kRowBytes, stream, static_cast<const uint8_t*>(packed), static_cast<const _Float16*>(B),
+                       static_cast<_Float16*>(out), units, per_batch, ldb, ldo, slab, N);
+    return static_cast<int>(hipGetLastError());
+}
+
+template<int NT>
+int launch_shared_b_nt(hipStream_t s, const void* packed, const void* B, void* out, int M, int N, int K, int split_k, int rb,
+                       int waves, long ldb, long ldo, long slab)
+{
+#define A24_CASE(RB_, W_)         \
+    if (rb == RB_ && waves == W_) \
+        return launch_shared_b<NT, RB_, W_>(s, packed, B, out, M, N, K, split_k, ldb, ldo, slab);
+    A24_CASE(2, 4) A24_CASE(2, 8) A24_CASE(4, 2) A24_CASE(4, 4) A24_CASE(4, 8) A24_CASE(8, 2) A24_CASE(8, 4)
+#undef A24_CASE
+    return static_cast<int>(hipErrorInvalidValue);
+}
+
 template<int NT, int RB, int W>
 int launch(hipStream_t stream, const void* packed, const void* B, void* out, int M, int N, int K, int split_k, long ldb,
            long ldo, long slab)
@@ -221,11 +393,20 @@ int launch_nt(hipStream_t s, const void* packed, const void* B, void* out, int M
 }  // namespace
 
 // Batch b of ceil((K/128)/split_k) units writes fp16 [N][ldo] to out + b * slab.  The caller has
-// checked: M % (16 * rb) == 0, K % 128 == 0, N in {8, 16, 32, 64}, no batch empty, pointers set.
+// checked: M % (16 * rb) == 0 (share_b: M % (16 * rb * waves) == 0), K % 128 == 0, N in {8, 16, 32, 64}, no batch empty, pointers set.
 extern "C" int a24_launch_spmm(void* stream, const void* packed, const void* B, void* out, int M, int N, int K,
-                               int split_k, int rb, int waves, long ldb, long ldo, long slab)
+                               int split_k, int rb, int waves, int share_b, long ldb, long ldo, long slab)
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (share_b) {  // waves own rows and share the activation tile through LDS
+        switch (N) {
+            case 8:
+            case 16: return launch_shared_b_nt<1>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab);
+            case 32: return launch_shared_b_nt<2>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab);
+            case 64: return launch_shared_b_nt<4>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab);
+            default: return static_cast<int>(hipErrorInvalidValue);
+        }
+    }
     switch (N) {
         case 8:
         case 16: return launch_nt<1>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab);

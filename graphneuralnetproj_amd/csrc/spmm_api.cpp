@@ -20,7 +20,7 @@ int tcsl_launch_copy(void* stream, void* dst, const void* src, long bytes);
 int tcsl_launch_encode_offsets(void* stream, const void* A, int M, int K, int* offsets);
 int tcsl_launch_encode_items(void* stream, const void* A, int M, int K, const int* offsets, void* items);
 int a24_launch_spmm(void* stream, const void* packed, const void* B, void* out, int M, int N, int K, int split_k, int rb,
-                    int waves, long ldb, long ldo, long slab);
+                    int waves, int share_b, long ldb, long ldo, long slab);
 int a24_side_begin(void* stream, void** side);
 int a24_side_end(void* stream, void* side);
 void* tcsl_event_create(void);
@@ -395,18 +395,19 @@ namespace {
 // Launch shape of the 2:4 kernel: row blocks per workgroup, waves per workgroup, split-K.
 struct A24Plan {
     int row_blocks, waves, split_k;
+    int share_b = 0;  // 0: the waves of a workgroup split K and add up; 1: they split rows and share the activation tile in LDS
 };
 
 A24Plan a24_default_plan(int M, int N, int K)
 {
-    // From a sweep on the OPT-30B shapes: as many rows per wave as the registers hold (a wave's
-    // activation fragments are shared by its row blocks), four waves per workgroup, and split-K
-    // until about two workgroups per compute unit exist (one for N >= 32).
-    A24Plan p{N == 64 ? 4 : 8, 4, 1};
-    const long groups = M / (16 * p.row_blocks);
-    const long target = N <= 16 ? 448 : 224;
+    // From a sweep on the OPT-30B shapes: workgroups of four waves with two row blocks each (128
+    // rows) that share the activation tile through LDS are the best or within 4 % of it for every
+    // token count, and split-K until about two workgroups per compute unit exist.
+    A24Plan p{2, 4, 1, 1};
+    (void)N;
+    const long groups = M / (16 * p.row_blocks * p.waves);
     const int units = K / a24::kUnitCols;
-    while (groups * p.split_k < target) {
+    while (groups * p.split_k < 448) {
         const int s2 = p.split_k * 2;
         const int per = (units + s2 - 1) / s2;
         if (per < 2 || static_cast<long>(per) * (s2 - 1) >= units)
@@ -416,7 +417,7 @@ A24Plan a24_default_plan(int M, int N, int K)
     return p;
 }
 
-bool a24_shape_ok(int M, int N, int K, int split_k, int row_blocks, int waves)
+bool a24_shape_ok(int M, int N, int K, int split_k, int row_blocks, int waves, int share_b = 0)
 {
     if (N != 8 && N != 16 && N != 32 && N != 64)
         return false;
@@ -428,6 +429,11 @@ bool a24_shape_ok(int M, int N, int K, int split_k, int row_blocks, int waves)
         return false;
     if (row_blocks < 1 || row_blocks > 8 || (row_blocks & (row_blocks - 1)) || waves < 1 || waves > 8)
         return false;
+    if (share_b) {  // the kernel table of this layout, and whole workgroups only
+        if (row_blocks < 2 || waves < 2 || row_blocks * waves < 8 || M % (16 * row_blocks * waves) != 0)
+            return false;
+        return true;
+    }
     if (N == 64 && (row_blocks == 8 || (row_blocks == 4 && waves == 8)))  // accumulators would not fit the registers
         return false;
     return true;
@@ -436,20 +442,21 @@ bool a24_shape_ok(int M, int N, int K, int split_k, int row_blocks, int waves)
 }  // namespace
 
 extern "C" int HeteroSparse_A1_Partials(void* stream, const void* Packed_A1, const void* B, void* Partials, int M, int N,
-                                        int K, int Split_K, int RowBlocks, int Waves)
+                                        int K, int Split_K, int RowBlocks, int Waves, int ShareB)
 {
-    A24Plan p{RowBlocks, Waves, Split_K};
+    A24Plan p{RowBlocks, Waves, Split_K, ShareB ? 1 : 0};
     if (RowBlocks == 0 || Waves == 0) {
         const A24Plan d = a24_default_plan(M > 0 ? M : 128, N, K > 0 ? K : 128);
         p.row_blocks = d.row_blocks;
         p.waves = d.waves;
+        p.share_b = d.share_b;
     }
-    if (!Packed_A1 || !B || !Partials || !a24_shape_ok(M, N, K, p.split_k, p.row_blocks, p.waves)) {
+    if (!Packed_A1 || !B || !Partials || !a24_shape_ok(M, N, K, p.split_k, p.row_blocks, p.waves, p.share_b)) {
         std::fprintf(stderr, "HeteroSparse_A1_Partials: unsupported call M=%d N=%d K=%d Split_K=%d (need M %% 128 == 0, K %% 128 == 0, N in {8,16,32,64}, no empty batch)\n",
                      M, N, K, Split_K);
         return tcsl_error_invalid_value();
     }
-    return a24_launch_spmm(stream, Packed_A1, B, Partials, M, N, K, p.split_k, p.row_blocks, p.waves, K, M,
+    return a24_launch_spmm(stream, Packed_A1, B, Partials, M, N, K, p.split_k, p.row_blocks, p.waves, p.share_b, K, M,
                            static_cast<long>(M) * N);
 }
 
@@ -470,7 +477,7 @@ extern "C" int HeteroSparse_SpMM_API(void* stream, const void* Packed_A1, const 
         return tcsl_error_unknown();
     }
     const A24Plan d = a24_shape_ok(M, N, K, Split_K_A1, 1, 1) ? a24_default_plan(M, N, K) : A24Plan{1, 1, 1};
-    if (!Packed_A1 || !B || !C || (residual && !TileOffsets_A2) || !a24_shape_ok(M, N, K, Split_K_A1, d.row_blocks, d.waves)
+    if (!Packed_A1 || !B || !C || (residual && !TileOffsets_A2) || !a24_shape_ok(M, N, K, Split_K_A1, d.row_blocks, d.waves, d.share_b)
         || (residual && (Split_K_A2 < 1 || Split_K_A2 > 65535)) || ((residual || Split_K_A1 > 1) && !Reduction_Workspace)
         || (Flags & ~HETERO_FLAG_TWO_STREAMS)) {
         std::fprintf(stderr, "HeteroSparse_SpMM_API: unsupported call M=%d N=%d K=%d Split_K=%d/%d (need M %% 128 == 0, K %% 128 == 0, no empty batch, non-null pointers)\n",
@@ -479,7 +486,7 @@ extern "C" int HeteroSparse_SpMM_API(void* stream, const void* Packed_A1, const 
     }
     const long mn = static_cast<long>(M) * N;
     if (!residual && Split_K_A1 == 1)  // the 2:4 kernel writes C itself
-        return a24_launch_spmm(stream, Packed_A1, B, C, M, N, K, 1, d.row_blocks, d.waves, K, M, mn);
+        return a24_launch_spmm(stream, Packed_A1, B, C, M, N, K, 1, d.row_blocks, d.waves, d.share_b, K, M, mn);
     int rc = 0;
     int slabs = Split_K_A1;
     if (residual) {
@@ -493,13 +500,13 @@ extern "C" int HeteroSparse_SpMM_API(void* stream, const void* Packed_A1, const 
         if (rc != 0)
             return rc;
         slabs += Split_K_A2;
-        rc = a24_launch_spmm(stream, Packed_A1, B, Reduction_Workspace, M, N, K, Split_K_A1, d.row_blocks, d.waves, K, M, mn);
+        rc = a24_launch_spmm(stream, Packed_A1, B, Reduction_Workspace, M, N, K, Split_K_A1, d.row_blocks, d.waves, d.share_b, K, M, mn);
         if (rc != 0)
             return rc;
         if ((rc = a24_side_end(stream, side)) != 0)
             return rc;
-    } else if ((rc = a24_launch_spmm(stream, Packed_A1, B, Reduction_Workspace, M, N, K, Split_K_A1, d.row_blocks, d.waves, K,
-                                     M, mn)) != 0) {
+    } else if ((rc = a24_launch_spmm(stream, Packed_A1, B, Reduction_Workspace, M, N, K, Split_K_A1, d.row_blocks, d.waves,
+                                     d.share_b, K, M, mn)) != 0) {
         return rc;
     }
     return tcsl_launch_reduce(stream, C, Reduction_Workspace, mn, 1, mn, slabs, 0);

@@ -161,7 +161,7 @@ def load_library():
     lib.HeteroSparse_SuggestSplitK.restype = ctypes.c_int
     lib.HeteroSparse_SuggestSplitK.argtypes = [ctypes.c_int] * 3
     lib.HeteroSparse_A1_Partials.restype = ctypes.c_int
-    lib.HeteroSparse_A1_Partials.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 6
+    lib.HeteroSparse_A1_Partials.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 7
     _lib = lib
     return lib
 
@@ -404,13 +404,13 @@ def HeteroSparse_SpMM_API(stream, Packed_A1, Compressed_A2, TileOffsets_A2, B, C
 
 
 def HeteroSparse_A1_Partials(stream, Packed_A1, B, Partials, M_Global, N_Global, K_Global, Split_K, RowBlocks=0,
-                             Waves=0):
+                             Waves=0, ShareB=0):
     """The 2:4 kernel alone, with a caller-chosen launch shape (0, 0 = the library's)."""
     lib = load_library()
     if stream is not None and not isinstance(stream, int):
         stream = stream.cuda_stream
     rc = lib.HeteroSparse_A1_Partials(ctypes.c_void_p(stream) if stream else None, _ptr(Packed_A1), _ptr(B),
-                                      _ptr(Partials), M_Global, N_Global, K_Global, Split_K, RowBlocks, Waves)
+                                      _ptr(Partials), M_Global, N_Global, K_Global, Split_K, RowBlocks, Waves, ShareB)
     if rc != 0:
         raise SpMMError("HeteroSparse_A1_Partials", rc, lib.SpMM_GetErrorString(rc).decode())
     return rc

@@ -298,11 +298,12 @@ SPMM_EXPORT int HeteroSparse_SuggestSplitK(int M_Global, int N_Global, int K_Glo
 /*
  * The 2:4 kernel alone: batch b of ceil((K/128)/Split_K) units writes fp16 A1*B partial sums to
  * Partials[b*M*N ..).  RowBlocks (16-row blocks per workgroup: 1, 2, 4, 8) and Waves (waves per
- * workgroup that split the batch: 1, 2, 4, 8) choose the launch shape; 0, 0 = the library's
- * choice.  hipErrorInvalidValue for shapes the kernel table does not hold.  For tuning and tests.
+ * workgroup: 1, 2, 4, 8) choose the launch shape; 0, 0 = the library's choice.  ShareB = 0: the
+ * waves of a workgroup split the batch's columns and add their sums up; ShareB = 1: they own
+ * RowBlocks row blocks each and share the activation tile through LDS (M % (16*RowBlocks*Waves) == 0).  hipErrorInvalidValue for shapes the kernel table does not hold.  For tuning and tests.
  */
 SPMM_EXPORT int HeteroSparse_A1_Partials(void* stream, const void* Packed_A1, const void* B, void* Partials, int M_Global,
-                                         int N_Global, int K_Global, int Split_K, int RowBlocks, int Waves);
+                                         int N_Global, int K_Global, int Split_K, int RowBlocks, int Waves, int ShareB);
 
 #ifdef __cplusplus
 }

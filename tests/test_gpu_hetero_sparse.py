@@ -38,12 +38,12 @@ def assert_close(C, ref):
     assert not bad.any(), f"{bad.sum()} elements out of tolerance, max err {err.max()} at {np.unravel_index(err.argmax(), err.shape)}"
 
 
-def run_a1(spmm, packed, B, M, N, K, split_k, rb=0, waves=0):
+def run_a1(spmm, packed, B, M, N, K, split_k, rb=0, waves=0, share_b=0):
     torch = _torch()
     d_p, d_B = _dev(packed), _dev(B)
     d_W = torch.full((split_k, N, M), float("nan"), dtype=torch.float16, device="cuda:0")
-    print(f"[gpu case] A1 partials M={M} N={N} K={K} split_k={split_k} rb={rb} waves={waves}", flush=True)
-    spmm.HeteroSparse_A1_Partials(torch.cuda.current_stream(), d_p, d_B, d_W, M, N, K, split_k, rb, waves)
+    print(f"[gpu case] A1 partials M={M} N={N} K={K} split_k={split_k} rb={rb} waves={waves} share_b={share_b}", flush=True)
+    spmm.HeteroSparse_A1_Partials(torch.cuda.current_stream(), d_p, d_B, d_W, M, N, K, split_k, rb, waves, share_b)
     torch.cuda.synchronize()
     return d_W.cpu().numpy()
 
@@ -98,6 +98,30 @@ def test_a1_launch_shapes_vs_oracle(spmm, oracle, N, rb, waves):
         for b in range(split_k):
             ref = oracle.gemm_f32(oracle.a24_unpack(packed, M, K), B, b * per * 128, min(K, (b + 1) * per * 128))
             assert_close(W[b], ref)
+
+
+@pytest.mark.parametrize("N", [8, 16, 32, 64])
+@pytest.mark.parametrize("rb,waves", [(2, 4), (2, 8), (4, 2), (4, 4), (4, 8), (8, 2), (8, 4)])
+def test_a1_shared_tile_shapes_vs_oracle(spmm, oracle, N, rb, waves):
+    """The layout whose waves own rows and share the activation tile through LDS."""
+    M, K = 512, 640  # five units: odd count, both buffers and both loop phases end a batch
+    A = spmm.synth_weights(M, K, 0.5, False, seed=N + rb + waves)
+    B = spmm.synth_activations(N, K, seed=78)
+    A1, _ = spmm.HeteroSparse_Decompose(A)
+    packed = spmm.HeteroSparse_PackA1(A1)
+    dense = oracle.a24_unpack(packed, M, K)
+    for split_k in (1, 2, 5):
+        W = run_a1(spmm, packed, B, M, N, K, split_k, rb, waves, 1)
+        per = -(-(K // 128) // split_k)
+        for b in range(split_k):
+            assert_close(W[b], oracle.gemm_f32(dense, B, b * per * 128, min(K, (b + 1) * per * 128)))
+
+
+def test_a1_shared_tile_rejects_partial_workgroups(spmm):
+    torch = _torch()
+    d = torch.zeros(1 << 16, dtype=torch.int32, device="cuda:0")
+    with pytest.raises(spmm.SpMMError):  # 128 rows are not a multiple of 16 * 4 * 4
+        spmm.HeteroSparse_A1_Partials(None, d, d, d, 128, 16, 128, 1, 4, 4, 1)
 
 
 @pytest.mark.parametrize("sparsity", [0.5, 0.7, 0.8, 0.95])
