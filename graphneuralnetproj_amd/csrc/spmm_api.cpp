@@ -132,6 +132,7 @@ struct CallOptions {
     void* ev_end = nullptr;
     const tcsl::LaunchPlan* forced = nullptr;
     bool adaptive_waves = false;  // with `forced`: launch it the way a planned call would be
+    int extra_slabs = 0;      // fused reduction only: slabs of an earlier launch, right behind this one's, to add as well
 };
 
 // fused_out != nullptr asks for the fused reduction; *fused says whether it was possible.
@@ -162,7 +163,8 @@ int launch_main(void* stream, const void* Compressed_A, const int* TileOffsets, 
     }
     return tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, out, M, N, K, Split_K, run.mode, run.waves, run.stage_b,
                             o.row_major ? 1 : 0, run.lds_bytes, ldb, ldo,
-                            relu && (Split_K == 1 || page >= 0) ? 1 : 0,  // slabs of partial sums are never clamped
+                            (relu && (Split_K == 1 || page >= 0) ? 1 : 0)  // slabs of partial sums are never clamped
+                                | (page >= 0 ? o.extra_slabs << 8 : 0),
                             page >= 0 ? fused_out : nullptr, static_cast<int>(ldc), page, dense_waves);
 }
 
@@ -488,26 +490,45 @@ extern "C" int HeteroSparse_SpMM_API(void* stream, const void* Packed_A1, const 
     if (!residual && Split_K_A1 == 1)  // the 2:4 kernel writes C itself
         return a24_launch_spmm(stream, Packed_A1, B, C, M, N, K, 1, d.row_blocks, d.waves, d.share_b, K, M, mn);
     int rc = 0;
-    int slabs = Split_K_A1;
-    if (residual) {
+    uint16_t* ws = static_cast<uint16_t*>(Reduction_Workspace);
+    if (!residual) {
+        rc = a24_launch_spmm(stream, Packed_A1, B, ws, M, N, K, Split_K_A1, d.row_blocks, d.waves, d.share_b, K, M, mn);
+        return rc != 0 ? rc : tcsl_launch_reduce(stream, C, ws, mn, 1, mn, Split_K_A1, 0);
+    }
+    // Slabs: the residual's Split_K_A2 first, the 2:4 part's Split_K_A1 behind them.
+    uint16_t* ws_a1 = ws + Split_K_A2 * mn;
+    bool fused = false;
+    if (Flags & HETERO_FLAG_TWO_STREAMS) {
         // On request the residual's kernel goes to a second stream, beside the 2:4 kernel.  Measured
-        // slower than one stream (two event waits cost more than the overlap gains), hence optional.
+        // slower than one stream (the two kernels compete, and two event waits cost more than the
+        // overlap gains), hence optional.
         void* side = stream;
-        if ((Flags & HETERO_FLAG_TWO_STREAMS) && (rc = a24_side_begin(stream, &side)) != 0)
+        if ((rc = a24_side_begin(stream, &side)) != 0)
             return rc;
-        rc = launch_main(side, Compressed_A2, TileOffsets_A2, B, static_cast<uint16_t*>(Reduction_Workspace) + slabs * mn, M,
-                         N, K, Split_K_A2, CallOptions{}, K, M, false, nullptr, 0, nullptr);
-        if (rc != 0)
+        CallOptions o;
+        o.separate_reduction = true;
+        if ((rc = launch_main(side, Compressed_A2, TileOffsets_A2, B, ws, M, N, K, Split_K_A2, o, K, M, false, nullptr, 0,
+                              nullptr)) != 0)
             return rc;
-        slabs += Split_K_A2;
-        rc = a24_launch_spmm(stream, Packed_A1, B, Reduction_Workspace, M, N, K, Split_K_A1, d.row_blocks, d.waves, d.share_b, K, M, mn);
-        if (rc != 0)
+        if ((rc = a24_launch_spmm(stream, Packed_A1, B, ws_a1, M, N, K, Split_K_A1, d.row_blocks, d.waves, d.share_b, K, M,
+                                  mn)) != 0)
             return rc;
         if ((rc = a24_side_end(stream, side)) != 0)
             return rc;
-    } else if ((rc = a24_launch_spmm(stream, Packed_A1, B, Reduction_Workspace, M, N, K, Split_K_A1, d.row_blocks, d.waves,
-                                     d.share_b, K, M, mn)) != 0) {
-        return rc;
+    } else {
+        // One stream: the 2:4 kernel first; the residual's kernel then adds everything up itself where
+        // its launch shape has the in-launch reduction (the last workgroup of a tile row sums that
+        // row's slabs, the 2:4 part's included), which saves the separate reduction kernel.
+        if ((rc = a24_launch_spmm(stream, Packed_A1, B, ws_a1, M, N, K, Split_K_A1, d.row_blocks, d.waves, d.share_b, K, M,
+                                  mn)) != 0)
+            return rc;
+        CallOptions o;
+        o.extra_slabs = Split_K_A1;
+        if ((rc = launch_main(stream, Compressed_A2, TileOffsets_A2, B, ws, M, N, K, Split_K_A2, o, K, M, false, C, M,
+                              &fused)) != 0)
+            return rc;
     }
-    return tcsl_launch_reduce(stream, C, Reduction_Workspace, mn, 1, mn, slabs, 0);
+    if (fused)
+        return 0;
+    return tcsl_launch_reduce(stream, C, ws, mn, 1, mn, Split_K_A1 + Split_K_A2, 0);
 }

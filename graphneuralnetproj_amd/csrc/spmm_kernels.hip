@@ -231,6 +231,8 @@ __device__ __forceinline__ void clear_tile(uint8_t* tile, int lane)
 // (csrc/Reduction_Kernel.cuh:36-46), so both paths give the same bits.  `counter` is the rows'
 // arrival count in device memory (zero between calls), `flag` one free LDS word, nthreads the
 // number of threads of the workgroup that are still there (the first nthreads).
+// Bits 8 and up of `relu` count further slabs that an earlier launch on the same stream left right
+// behind this launch's own Split_K (the 2:4 part's partial sums); they are added after them.
 __device__ __forceinline__ void fused_reduction_tail(const _Float16* __restrict__ slabs, _Float16* __restrict__ C, int M,
                                                      int N, int ldc, int split_k, int relu, int row0, int nrows,
                                                      unsigned int* counter, unsigned int* flag, int nthreads)
@@ -243,6 +245,8 @@ __device__ __forceinline__ void fused_reduction_tail(const _Float16* __restrict_
     __syncthreads();
     if (*flag != static_cast<unsigned int>(split_k - 1))
         return;
+    split_k += relu >> 8;
+    relu &= 0xff;
     nrows = nrows < M - row0 ? nrows : M - row0;
     const int per_tok = nrows / 8;
     const size_t slab = (size_t)M * N;
@@ -950,6 +954,8 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
 // ldb, ldo: token strides of B and of the output in elements (column-major; multiples of 8).
 // fuse_page >= 0: out = Split_K dense slabs, and the kernel itself reduces them into fused_out
 // (token stride ldc), counting arrivals on that page of counters; at most 4096 row groups.
+// relu: bit 0 clamps final results at zero; with fuse_page >= 0, bits 8 and up = number of further
+// slabs behind the Split_K of this launch that the fused reduction adds as well.
 // dense_waves (mode 1; 0 = off): of the `waves` launched, only this many work on a unit whose
 // tiles average 340 vectors or more (six on sparser units); the kernel looks at each unit's own offsets.
 extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offsets, const void* B, void* out, int M,
@@ -964,7 +970,7 @@ extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offs
         return static_cast<int>(hipErrorInvalidValue);
     if (fuse_page >= 0) {
         const long groups = mode ? M / kTileRows : (M / kTileRows + waves - 1) / waves;
-        if (fuse_page >= kCounterPages || groups > kCountersPerPage || row_major || split_k < 2 || !fused_out)
+        if (fuse_page >= kCounterPages || groups > kCountersPerPage || row_major || split_k + (relu >> 8) < 2 || !fused_out)
             return static_cast<int>(hipErrorInvalidValue);
     }
 #define TCSL_GO(NB, HALF, BLDS, KS, RM, MAXW) \

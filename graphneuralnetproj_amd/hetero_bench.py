@@ -63,12 +63,18 @@ def main():
         c = args.copies
         d_items, d_offs = [up(items) for _ in range(c)], [up(offs) for _ in range(c)]
         d_p, d_i2, d_o2 = [up(packed) for _ in range(c)], [up(items2) for _ in range(c)], [up(offs2) for _ in range(c)]
+        first = True
         for N in [int(x) for x in args.n.split(",")]:
             B = up(G.synth_activations(N, K, seed=1))
             C = torch.empty((N, M), dtype=torch.float16, device=dev)
             s0 = G.SpMM_SuggestSplitK(M, N, K)
             s1 = G.HeteroSparse_SuggestSplitK(M, N, K)
             W = torch.empty((s0 + s1 + 64, N, M), dtype=torch.float16, device=dev)
+            if first:  # the host work above let the clocks drop: bring them back before timing anything
+                for i in range(1500):
+                    G.SpMM_SplitK_API(st, None, d_items[i % c], d_offs[i % c], B, C, M, N, K, W, s0)
+                torch.cuda.synchronize()
+                first = False
             t_csl = time_us(lambda i: G.SpMM_SplitK_API(st, None, d_items[i % c], d_offs[i % c], B, C, M, N, K, W, s0))
             t_a1 = time_us(lambda i: G.HeteroSparse_A1_Partials(st, d_p[i % c], B, W, M, N, K, s1))
             t_h = time_us(lambda i: G.HeteroSparse_SpMM_API(st, d_p[i % c], d_i2[i % c], d_o2[i % c], B, C, M, N, K, W, s1, s0))
