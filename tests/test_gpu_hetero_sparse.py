@@ -183,3 +183,61 @@ def test_hybrid_full_size_sampled_rows(spmm, oracle):
     tol = 2e-2 if exact else 4e-2
     assert np.isfinite(Cs).all()
     assert (np.abs(Cs.astype(np.float32) - lin) <= tol + tol * np.abs(lin)).all()
+
+
+@pytest.mark.parametrize("flags_name", ["one_stream", "two_streams"])
+def test_hybrid_hip_graph_replays_match_eager(spmm, oracle, flags_name):
+    """The hybrid call captured into a HIP graph and replayed, with eager calls in between, gives
+    the eager bits every time (the library records kernels and event edges only, no memset nodes)."""
+    torch = _torch()
+    flags = spmm.HETERO_FLAG_TWO_STREAMS if flags_name == "two_streams" else 0
+    M, K, N = 1024, 1024, 16
+    A = spmm.synth_weights(M, K, 0.6, False, seed=31)
+    A1, A2 = spmm.HeteroSparse_Decompose(A)
+    d_p = _dev(spmm.HeteroSparse_PackA1(A1))
+    items, offsets = spmm.InitSparseMatrixA_API(A2)
+    d_items, d_offs = _dev(items), _dev(offsets)
+    d_B = _dev(spmm.synth_activations(N, K, seed=32))
+    d_C = torch.zeros((N, M), dtype=torch.float16, device="cuda:0")
+    d_W = torch.zeros((6, N, M), dtype=torch.float16, device="cuda:0")
+
+    def call(stream):
+        spmm.HeteroSparse_SpMM_API(stream, d_p, d_items, d_offs, d_B, d_C, M, N, K, d_W, 2, 4, flags)
+
+    print(f"[gpu case] graph capture of the hybrid call, {flags_name}", flush=True)
+    call(torch.cuda.current_stream())  # eager reference; creates the library's second stream before capture
+    torch.cuda.synchronize()
+    want = d_C.clone()
+    assert_close(want.cpu().numpy(), oracle.gemm_f32(A, spmm.synth_activations(N, K, seed=32)))
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        call(torch.cuda.current_stream())  # the capturing stream gets its own second stream first
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            call(torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    for rep in range(3):
+        d_C.zero_()
+        d_W.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(d_C, want), f"replay {rep} differs from the eager result"
+        d_C.zero_()
+        call(torch.cuda.current_stream())
+        torch.cuda.synchronize()
+        assert torch.equal(d_C, want)
+
+
+def test_a1_full_size_ffn2_n64_sampled_rows(spmm, oracle):
+    """OPT-30B FFN2 (7168 x 28672) as a 2:4 weight, N = 64, the library's own launch: sampled rows."""
+    M, K, N = 7168, 28672, 64
+    A = spmm.synth_weights(M, K, 0.6, False, seed=41)
+    A1, _ = spmm.HeteroSparse_Decompose(A)
+    packed = spmm.HeteroSparse_PackA1(A1)
+    B = spmm.synth_activations(N, K, seed=42)
+    s1 = spmm.HeteroSparse_SuggestSplitK(M, N, K)
+    assert s1 > 1
+    C = run_hybrid(spmm, packed, None, None, B, M, N, K, s1, 0)
+    rows = np.sort(np.random.default_rng(1).choice(M, 256, replace=False))
+    assert_close(C[:, rows], oracle.gemm_f32(np.ascontiguousarray(A1[rows]), B))
