@@ -416,6 +416,90 @@ extern "C" int a24_launch_spmm(void* stream, const void* packed, const void* B, 
     }
 }
 
+// Split and pack on the GPU: the same bits as the host's decompose + pack (a24_pack.cpp), for
+// weights that are already in device memory.  One thread per lane of a record: it reads its row's
+// 4 x 8 columns of the unit, keeps the first two kept values of every group of four
+// (kernel_benchmark/spmm_decompose.h:12-51) in the record and writes the others to the dense
+// residual (when asked for one), zero elsewhere.
+__global__ __launch_bounds__(256) void a24_split_pack_kernel(const uint16_t* __restrict__ A, uint8_t* __restrict__ packed,
+                                                             uint16_t* __restrict__ residual, int K, int units,
+                                                             long records)
+{
+    const long id = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long record = id >> 6;
+    if (record >= records)
+        return;
+    const int L = static_cast<int>(id & 63);
+    const long rb = record / units;
+    const int u = static_cast<int>(record - rb * units);
+    const size_t row = (size_t)(rb * 16 + (L & 15)) * K + (size_t)u * 128 + (L >> 4) * 8;
+    uint8_t* rec = packed + (size_t)record * kRecordBytes;
+    typedef unsigned short u16x8 __attribute__((ext_vector_type(8)));
+    unsigned word = 0;
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        const u16x8 in = *reinterpret_cast<const u16x8*>(A + row + s * 32);
+        u16x8 rest = {0, 0, 0, 0, 0, 0, 0, 0};
+        unsigned short val[4];
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            int pos[2] = {0, 1}, n = 0;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const unsigned short v = in[half * 4 + e];
+                if ((v & 0x7fffu) != 0) {  // compares unequal to zero as a float: NaN counts, -0 does not
+                    if (n < 2)
+                        pos[n] = e;
+                    else
+                        rest[half * 4 + e] = v;
+                    n++;
+                }
+            }
+            unsigned short v0 = 0, v1 = 0;
+            if (n >= 2) {
+                v0 = in[half * 4 + pos[0]];
+                v1 = in[half * 4 + pos[1]];
+            } else if (n == 1) {
+                if (pos[0] == 3) {  // the free slot goes before it
+                    v1 = in[half * 4 + 3];
+                    pos[0] = 2;
+                    pos[1] = 3;
+                } else {
+                    v0 = in[half * 4 + pos[0]];
+                    pos[1] = 3;
+                }
+            } else {
+                pos[0] = 0;
+                pos[1] = 1;
+            }
+            val[half * 2] = v0;
+            val[half * 2 + 1] = v1;
+            word |= static_cast<unsigned>(pos[0]) << (8 * s + 4 * half) | static_cast<unsigned>(pos[1]) << (8 * s + 4 * half + 2);
+        }
+        typedef unsigned short u16x4 __attribute__((ext_vector_type(4)));
+        const u16x4 out = {val[0], val[1], val[2], val[3]};
+        *reinterpret_cast<u16x4*>(rec + (s >> 1) * 1024 + L * 16 + (s & 1) * 8) = out;
+        if (residual)
+            *reinterpret_cast<u16x8*>(residual + row + s * 32) = rest;
+    }
+    *reinterpret_cast<unsigned*>(rec + 2048 + L * 4) = word;
+}
+
+// A: row-major M x K fp16 in device memory (M % 16 == 0, K % 128 == 0, checked by the caller);
+// residual may be null.
+extern "C" int a24_launch_split_pack(void* stream, const void* A, void* packed, void* residual, int M, int K)
+{
+    const int units = K / 128;
+    const long records = static_cast<long>(M / 16) * units;
+    const long blocks = (records * 64 + 255) / 256;
+    if (blocks < 1 || blocks > 0x7fffffffL)
+        return static_cast<int>(hipErrorInvalidValue);
+    hipLaunchKernelGGL(a24_split_pack_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint16_t*>(A), static_cast<uint8_t*>(packed), static_cast<uint16_t*>(residual), K,
+                       units, records);
+    return static_cast<int>(hipGetLastError());
+}
+
 // A second stream per caller stream, so that the residual's Tiled-CSL kernel can run beside the 2:4
 // kernel (the reference gives them two streams as well, kernel_benchmark/spmm_test.cu:459-461).
 // Default priority, created on first use, kept until the process ends; at most 32 caller

@@ -21,6 +21,7 @@ int tcsl_launch_encode_offsets(void* stream, const void* A, int M, int K, int* o
 int tcsl_launch_encode_items(void* stream, const void* A, int M, int K, const int* offsets, void* items);
 int a24_launch_spmm(void* stream, const void* packed, const void* B, void* out, int M, int N, int K, int split_k, int rb,
                     int waves, int share_b, long ldb, long ldo, long slab);
+int a24_launch_split_pack(void* stream, const void* A, void* packed, void* residual, int M, int K);
 int a24_side_begin(void* stream, void** side);
 int a24_side_end(void* stream, void* side);
 void* tcsl_event_create(void);
@@ -390,6 +391,15 @@ extern "C" long HeteroSparse_PackedBytes(int M, int K)
 extern "C" int HeteroSparse_PackA1(const uint16_t* A1_h, int M, int K, void* Packed_h)
 {
     return a24::pack(A1_h, M, K, static_cast<uint8_t*>(Packed_h));
+}
+
+extern "C" int HeteroSparse_DeviceSplitPack(void* stream, const void* A_d, int M, int K, void* Packed_A1_d, void* A2_d)
+{
+    if (!A_d || !Packed_A1_d || M <= 0 || K <= 0 || M % a24::kRows != 0 || K % a24::kUnitCols != 0) {
+        std::fprintf(stderr, "HeteroSparse_DeviceSplitPack: need M %% 16 == 0, K %% 128 == 0 and non-null pointers (M=%d K=%d)\n", M, K);
+        return tcsl_error_invalid_value();
+    }
+    return a24_launch_split_pack(stream, A_d, Packed_A1_d, A2_d, M, K);
 }
 
 namespace {

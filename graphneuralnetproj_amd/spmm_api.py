@@ -56,6 +56,7 @@ EXPORTED_SYMBOLS = (
     "HeteroSparse_SpMM_API",
     "HeteroSparse_SuggestSplitK",
     "HeteroSparse_A1_Partials",
+    "HeteroSparse_DeviceSplitPack",
 )
 
 
@@ -160,6 +161,9 @@ def load_library():
     lib.HeteroSparse_SpMM_API.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int] * 3 + [ctypes.c_void_p] + [ctypes.c_int] * 3
     lib.HeteroSparse_SuggestSplitK.restype = ctypes.c_int
     lib.HeteroSparse_SuggestSplitK.argtypes = [ctypes.c_int] * 3
+    lib.HeteroSparse_DeviceSplitPack.restype = ctypes.c_int
+    lib.HeteroSparse_DeviceSplitPack.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
+                                                 ctypes.c_void_p, ctypes.c_void_p]
     lib.HeteroSparse_A1_Partials.restype = ctypes.c_int
     lib.HeteroSparse_A1_Partials.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 7
     _lib = lib
@@ -414,3 +418,26 @@ def HeteroSparse_A1_Partials(stream, Packed_A1, B, Partials, M_Global, N_Global,
     if rc != 0:
         raise SpMMError("HeteroSparse_A1_Partials", rc, lib.SpMM_GetErrorString(rc).decode())
     return rc
+
+
+def split_pack_on_device(A_d, want_residual=True, stream=None):
+    """2:4 records (uint8 tensor) and dense residual (fp16 tensor, or None) of a torch CUDA fp16 matrix,
+    made on the GPU; same bits as HeteroSparse_Decompose + HeteroSparse_PackA1."""
+    import torch
+
+    lib = load_library()
+    M, K = A_d.shape
+    if A_d.dtype != torch.float16 or not A_d.is_contiguous():
+        raise TypeError("expected a contiguous float16 CUDA tensor")
+    size = lib.HeteroSparse_PackedBytes(M, K)
+    if size < 0:
+        raise SpMMError("HeteroSparse_PackedBytes", int(size))
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    packed = torch.empty(size, dtype=torch.uint8, device=A_d.device)
+    residual = torch.empty_like(A_d) if want_residual else None
+    rc = lib.HeteroSparse_DeviceSplitPack(ctypes.c_void_p(stream.cuda_stream) if stream.cuda_stream else None, _ptr(A_d),
+                                          M, K, _ptr(packed), _ptr(residual))
+    if rc != 0:
+        raise SpMMError("HeteroSparse_DeviceSplitPack", rc, lib.SpMM_GetErrorString(rc).decode())
+    return packed, residual

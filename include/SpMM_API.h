@@ -272,6 +272,16 @@ SPMM_EXPORT long HeteroSparse_PackedBytes(int M, int K);
 SPMM_EXPORT int HeteroSparse_PackA1(const uint16_t* A1_h, int M, int K, void* Packed_h);
 
 /*
+ * Split and pack on the GPU, for a weight that is already in device memory (row-major M x K fp16 at
+ * A_d, M % 16 == 0, K % 128 == 0): Packed_A1_d receives the records (HeteroSparse_PackedBytes bytes),
+ * A2_d, if not NULL, the dense residual (M*K fp16, zero where nothing is left), ready for
+ * SpMM_DeviceEncodeOffsets / SpMM_DeviceEncodeItems.  Same bits as HeteroSparse_Decompose followed by
+ * HeteroSparse_PackA1.  Only enqueues a kernel on `stream`; returns a hipError_t value.  The reference
+ * does both steps on one host thread (kernel_benchmark/spmm_test.cu:285-330).
+ */
+SPMM_EXPORT int HeteroSparse_DeviceSplitPack(void* stream, const void* A_d, int M, int K, void* Packed_A1_d, void* A2_d);
+
+/*
  * C = A1*B + A2*B on the GPU; the counterpart of this checkout's 13-argument SpMM_SplitK_API call
  * followed by its residual kernel and reduction (kernel_benchmark/spmm_test.cu:462-560).
  * Packed_A1: device copy of the records; Compressed_A2 / TileOffsets_A2: device Tiled-CSL of the

@@ -241,3 +241,49 @@ def test_a1_full_size_ffn2_n64_sampled_rows(spmm, oracle):
     C = run_hybrid(spmm, packed, None, None, B, M, N, K, s1, 0)
     rows = np.sort(np.random.default_rng(1).choice(M, 256, replace=False))
     assert_close(C[:, rows], oracle.gemm_f32(np.ascontiguousarray(A1[rows]), B))
+
+
+@pytest.mark.parametrize("M,K,sparsity", [(16, 128, 0.5), (256, 640, 0.2), (1024, 2048, 0.8), (128, 128, 1.0), (128, 256, 0.0)])
+def test_device_split_pack_equals_host(spmm, oracle, M, K, sparsity):
+    """The GPU's split + pack against the host's (itself pinned by the oracle), bit for bit,
+    including -0, NaN, denormal and infinity patterns; then the device-made pair through the hybrid."""
+    torch = _torch()
+    A = spmm.synth_weights(M, K, sparsity, False, seed=M + K)
+    A.view(np.uint16)[0, :8] = [0x8000, 0x7E00, 0x0001, 0x3C00, 0xFC00, 0x8001, 0, 0x7C00]
+    A1, A2 = oracle.decompose(A)
+    want = spmm.HeteroSparse_PackA1(A1)
+    d_A = torch.from_numpy(A.view(np.int16).copy()).to("cuda:0").view(torch.float16)
+    print(f"[gpu case] device split+pack M={M} K={K} sparsity={sparsity}", flush=True)
+    packed, residual = spmm.split_pack_on_device(d_A)
+    torch.cuda.synchronize()
+    assert np.array_equal(packed.cpu().numpy(), want)
+    assert np.array_equal(residual.cpu().numpy().view(np.uint16), A2.view(np.uint16))
+    packed_only, none = spmm.split_pack_on_device(d_A, want_residual=False)
+    torch.cuda.synchronize()
+    assert none is None and torch.equal(packed_only, packed)
+
+
+def test_device_pipeline_dense_to_hybrid(spmm, oracle):
+    """Dense weight on the GPU -> records + residual -> Tiled-CSL of the residual -> product, no host step."""
+    torch = _torch()
+    M, K, N = 512, 1024, 16
+    A = spmm.synth_weights(M, K, 0.6, False, seed=55)
+    A.view(np.uint16)[A.view(np.uint16) == 0x8000] = 0
+    B = spmm.synth_activations(N, K, seed=56)
+    d_A = torch.from_numpy(A.view(np.int16).copy()).to("cuda:0").view(torch.float16)
+    packed, residual = spmm.split_pack_on_device(d_A)
+    items, offs = spmm.encode_on_device(residual)
+    d_B = _dev(B)
+    d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device="cuda:0")
+    d_W = torch.empty((4, N, M), dtype=torch.float16, device="cuda:0")
+    print("[gpu case] device pipeline dense -> hybrid", flush=True)
+    spmm.HeteroSparse_SpMM_API(torch.cuda.current_stream(), packed, items, offs, d_B, d_C, M, N, K, d_W, 2, 2)
+    torch.cuda.synchronize()
+    assert_close(d_C.cpu().numpy(), oracle.gemm_f32(A, B))
+
+
+def test_device_split_pack_rejects_bad_shapes(spmm):
+    torch = _torch()
+    d = torch.zeros((16, 64), dtype=torch.float16, device="cuda:0")
+    with pytest.raises(spmm.SpMMError):
+        spmm.split_pack_on_device(d)
