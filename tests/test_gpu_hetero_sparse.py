@@ -287,3 +287,18 @@ def test_device_split_pack_rejects_bad_shapes(spmm):
     d = torch.zeros((16, 64), dtype=torch.float16, device="cuda:0")
     with pytest.raises(spmm.SpMMError):
         spmm.split_pack_on_device(d)
+
+
+@pytest.mark.parametrize("N", [16, 64])
+def test_hybrid_with_row_sharing_residual_launch(spmm, oracle, N):
+    """A shape whose residual launch is of the row-sharing kind, which has no in-launch reduction:
+    the hybrid must fall back to the separate reduction kernel over all slabs."""
+    M, K, s1, s2 = 16384, 512, 2, 3
+    assert spmm.SpMM_PlanLaunch(M, N, K, s2)["mode"] == 0
+    A = spmm.synth_weights(M, K, 0.6, False, seed=71 + N)
+    A1, A2 = spmm.HeteroSparse_Decompose(A)
+    packed = spmm.HeteroSparse_PackA1(A1)
+    items, offsets = spmm.InitSparseMatrixA_API(A2)
+    B = spmm.synth_activations(N, K, seed=72)
+    C = run_hybrid(spmm, packed, items, offsets, B, M, N, K, s1, s2)
+    assert_close(C, oracle.gemm_f32(A, B))
