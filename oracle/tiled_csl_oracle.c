@@ -29,7 +29,7 @@
  *   half conversions     - exhaustive comparison with numpy float16.
  *   oracle_decompose     - bit-compared with the reference's own decompose()
  *                          compiled from kernel_benchmark/spmm_decompose.h:12-51
- *                          (oracle/_ref); A1 + A2 == A with disjoint supports; at
+ *                          (oracle/_ref) and with committed golden vectors made by it; A1 + A2 == A with disjoint supports; at
  *                          most two kept values per group of four in A1; hand cases.
  *   oracle_a24_unpack    - reader of this build's 2:4 record layout (the reference's
  *                          own on-device form, csrc/SpMM_API.cu:1127-1553, is made for

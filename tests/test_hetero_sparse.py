@@ -1,6 +1,7 @@
 """CPU tests of the 2:4 + residual split and of the 2:4 record packer.
 
-decompose() is pinned three ways: the oracle against the reference's own function compiled
+decompose() is pinned four ways: committed golden vectors written by the reference's own
+function (tests/golden/decompose_small.npz), the oracle against that function compiled
 from kernel_benchmark/spmm_decompose.h:12-51 (oracle/_ref, where that build ran), hand-made
 groups whose answer is read off the reference's loop, and the properties the split must have.
 The product's HeteroSparse_Decompose is then compared with the oracle bit for bit.
@@ -8,10 +9,29 @@ The record layout is this build's own (the reference's is made for NVIDIA's mma.
 oracle's reader is pinned by records built by hand here, byte by byte, and the packer by
 unpack(pack(A1)) == A1.
 """
+import os
+
 import numpy as np
 import pytest
 
 H = np.float16
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "decompose_small.npz")
+
+
+def golden_cases():
+    z = np.load(GOLD)
+    names = sorted({k.rsplit(".", 1)[0] for k in z.files})
+    return [(n, z[n + ".A"], z[n + ".A1"], z[n + ".A2"]) for n in names]
+
+
+@pytest.mark.parametrize("name,A,A1,A2", golden_cases(), ids=[c[0] for c in golden_cases()])
+def test_decompose_matches_reference_golden(oracle, spmm, name, A, A1, A2):
+    """Committed outputs of the reference's own decompose() (tests/golden/make_golden.py): the oracle
+    and the product must both reproduce them bit for bit, with or without the reference build at hand."""
+    o1, o2 = oracle.decompose(A)
+    assert np.array_equal(o1.view(np.uint16), A1) and np.array_equal(o2.view(np.uint16), A2)
+    p1, p2 = spmm.HeteroSparse_Decompose(A)
+    assert np.array_equal(p1.view(np.uint16), A1) and np.array_equal(p2.view(np.uint16), A2)
 
 
 def _rand_sparse(rng, M, K, keep):
