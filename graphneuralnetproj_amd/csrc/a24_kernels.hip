@@ -1,13 +1,16 @@
-// gfx950 kernel for the 2:4 part of a weight: C[n][m] (+ split-K slabs) = A1 * B with A1 held as
+// gfx950 kernels for the 2:4 part of a weight: C[n][m] (+ split-K slabs) = A1 * B with A1 held as
 // records in sparse-MFMA operand order (layout: a24_format.h).  The reference runs this part on
 // NVIDIA's mma.sp (csrc/SpMM_Kernel.cuh:293-735 with csrc/MMA_PTX.cuh:195-210); nothing of that
 // is reused.  Here a wave loads values and positions straight into the registers that
-// v_smfmac_f32_16x16x32_f16 reads -- no LDS staging, no scatter -- and the activation fragments
-// come from the L2 in the same operand order as in the Tiled-CSL kernel.
+// v_smfmac_f32_16x16x32_f16 reads: no LDS staging of the weights, no scatter.
 //
-// Work split: a workgroup owns RB consecutive 16-row blocks of one split-K batch; its W waves
-// cut the batch's 128-column units among themselves, keep RB x N/16 accumulator tiles each, and
-// add them up through LDS in wave order at the end (fp32, one rounding to fp16).
+// Two work splits.  a24_spmm_kernel: a workgroup owns RB consecutive 16-row blocks of one split-K
+// batch; its W waves cut the batch's 128-column units among themselves, keep RB x N/16
+// accumulator tiles each, fetch their activation fragments from the L2 in operand order, and add
+// up through LDS in wave order at the end (fp32, one rounding to fp16).
+// a24_spmm_shared_b_kernel (the default launch): the waves own rows instead and share each unit's
+// activation tile through LDS.  Also here: the split + pack on the GPU, and the second stream
+// that the two-stream form of the hybrid call uses.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -184,7 +187,7 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_kernel(const uint8_t* __res
     }
 }
 
-// The other work split, for wide token counts: the W waves of a workgroup own RB row blocks each
+// The other work split, the library's default: the W waves of a workgroup own RB row blocks each
 // (16 * RB * W rows per workgroup) and walk the batch's units together.  The unit's activation
 // tile (n_tokens x 128 fp16) is fetched once per workgroup with full-line loads, kept in LDS
 // (two buffers, rows padded to 272 bytes so that the sixteen lanes of a quarter wave read sixteen

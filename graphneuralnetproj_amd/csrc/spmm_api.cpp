@@ -1,6 +1,7 @@
 // Host logic behind the C ABI declared in include/SpMM_API.h: argument
 // checking, the split-K plan and the order of launches.  Plain C++; the GPU is
-// reached only through the tcsl_* launchers of spmm_kernels.hip.
+// reached only through the tcsl_* launchers of spmm_kernels.hip and
+// tiled_csl_encode_device.hip and the a24_* launchers of a24_kernels.hip.
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
