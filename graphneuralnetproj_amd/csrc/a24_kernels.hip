@@ -15,6 +15,7 @@
 #include <stdint.h>
 
 #include <mutex>
+#include <type_traits>
 
 namespace {
 
@@ -25,6 +26,14 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWave = 64;
 constexpr int kRecordBytes = 2304;
+constexpr int kGroupBlocks = 8;                             // records of eight row blocks are stored together, unit by unit
+constexpr int kUnitStride = kGroupBlocks * kRecordBytes;    // bytes between a row block's records of two consecutive units
+
+// First record (unit 0) of 16-row block rb.
+__device__ __forceinline__ const uint8_t* block_records(const uint8_t* packed, int rb, int units)
+{
+    return packed + ((size_t)(rb / kGroupBlocks) * units * kGroupBlocks + rb % kGroupBlocks) * kRecordBytes;
+}
 
 struct AFrag {      // one record's share of a lane
     u32x4 v[2];     // steps 0,1 and steps 2,3: four fp16 values each
@@ -43,6 +52,36 @@ __device__ __forceinline__ AFrag load_a(const uint8_t* rec, int lane)
     a.v[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(rec + 1024 + lane * 16));
     a.idx = __builtin_nontemporal_load(reinterpret_cast<const unsigned*>(rec + 2048 + lane * 4));
     return a;
+}
+
+// The shared-tile kernel issues its loads from inline assembly and waits for them by hand: left
+// to itself the compiler sinks a prefetch to the block that first uses it and waits for every
+// load at the loop's joins, so no unit's loads ever overlap another unit's multiplication.  The
+// compiler does not know that these registers are written later; the source keeps every register
+// of a load untouched until the wait that covers it (the build checks that on the generated code).
+__device__ __forceinline__ AFrag issue_a(const uint8_t* rec_lane, const uint8_t* idx_lane)
+{
+    AFrag a;
+    asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(a.v[0]) : "v"(rec_lane));
+    asm volatile("global_load_dwordx4 %0, %1, off offset:1024 nt" : "=v"(a.v[1]) : "v"(rec_lane));
+    asm volatile("global_load_dword %0, %1, off offset:2048 nt" : "=v"(a.idx) : "v"(idx_lane));
+    return a;
+}
+__device__ __forceinline__ u32x4 issue_b(const _Float16* p)
+{
+    u32x4 r;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r) : "v"(p));
+    return r;
+}
+template<int N>
+__device__ __forceinline__ void wait_loads()  // at most N loads stay in flight (they complete in order)
+{
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N < 63 ? N : 63) : "memory");
+}
+template<typename T>
+__device__ __forceinline__ void settle(T& x)  // the register's value is the one that landed, from here on
+{
+    asm volatile("" : "+v"(x));
 }
 
 template<int NT>
@@ -102,7 +141,7 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_kernel(const uint8_t* __res
     const uint8_t* rec[RB];
 #pragma unroll
     for (int r = 0; r < RB; r++)
-        rec[r] = packed + ((size_t)(blockIdx.x * RB + r) * units) * kRecordBytes;
+        rec[r] = block_records(packed, blockIdx.x * RB + r, units);
     const _Float16* tok[NT];
 #pragma unroll
     for (int t = 0; t < NT; t++) {
@@ -125,13 +164,13 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_kernel(const uint8_t* __res
         load_b<NT>(f0, tok, u);
 #pragma unroll
         for (int r = 0; r < RB; r++)
-            a0[r] = load_a(rec[r] + (size_t)u * kRecordBytes, lane);
+            a0[r] = load_a(rec[r] + (size_t)u * kUnitStride, lane);
         while (true) {
             if (u + 1 < u1) {
                 load_b<NT>(f1, tok, u + 1);
 #pragma unroll
                 for (int r = 0; r < RB; r++)
-                    a1[r] = load_a(rec[r] + (size_t)(u + 1) * kRecordBytes, lane);
+                    a1[r] = load_a(rec[r] + (size_t)(u + 1) * kUnitStride, lane);
             }
             multiply<NT, RB>(acc, a0, f0);
             if (++u >= u1)
@@ -140,7 +179,7 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_kernel(const uint8_t* __res
                 load_b<NT>(f0, tok, u + 1);
 #pragma unroll
                 for (int r = 0; r < RB; r++)
-                    a0[r] = load_a(rec[r] + (size_t)(u + 1) * kRecordBytes, lane);
+                    a0[r] = load_a(rec[r] + (size_t)(u + 1) * kUnitStride, lane);
             }
             multiply<NT, RB>(acc, a1, f1);
             if (++u >= u1)
@@ -217,16 +256,14 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
     const uint8_t* rec[RB];
 #pragma unroll
     for (int r = 0; r < RB; r++)
-        rec[r] = packed + ((size_t)(block0 + r) * units) * kRecordBytes;
+        rec[r] = block_records(packed, block0 + r, units);
     // this thread's chunks of the activation tile: token c / 16, columns (c % 16) * 8 .. + 8
     const _Float16* src[CH];
     int dst[CH];
-    bool mine[CH];
 #pragma unroll
     for (int i = 0; i < CH; i++) {
         const int c = tid + i * kThreads;
-        mine[i] = c < n_tokens * 16;
-        const int n = mine[i] ? c >> 4 : 0;
+        const int n = c < n_tokens * 16 ? c >> 4 : 0;
         src[i] = B + (size_t)n * ldb + (c & 15) * 8;
         dst[i] = n * kRowBytes + (c & 15) * 16;
     }
@@ -246,18 +283,36 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
         for (int t = 0; t < NT; t++)
             acc[r][t] = float4v{0.f, 0.f, 0.f, 0.f};
 
-    u32x4 stage[CH];
-    auto fetch_b = [&](int u) {
-#pragma unroll
-        for (int i = 0; i < CH; i++)
-            if (mine[i])
-                stage[i] = *reinterpret_cast<const u32x4*>(src[i] + (size_t)u * 128);
+    // Three rotating sets of "unit registers": the records of RB row blocks and this thread's chunks
+    // of the activation tile.  (A thread beyond the tile's last chunk repeats one of token 0's: the
+    // same bytes to the same place, so that every thread issues the same number of loads.)
+    struct UnitRegs {
+        AFrag a[RB];
+        u32x4 stage[CH];
     };
-    auto store_b = [&](int buf) {
+    constexpr int kLoadsA = 3 * RB;      // loads of one unit's records per lane
+    auto issue_unit = [&](UnitRegs& x, int unit) {  // activation chunks first: they are needed first
 #pragma unroll
         for (int i = 0; i < CH; i++)
-            if (mine[i])
-                *reinterpret_cast<u32x4*>(tile + buf * kBuf + dst[i]) = stage[i];
+            x.stage[i] = issue_b(src[i] + (size_t)unit * 128);
+#pragma unroll
+        for (int r = 0; r < RB; r++)
+            x.a[r] = issue_a(rec[r] + (size_t)unit * kUnitStride + lane * 16, rec[r] + (size_t)unit * kUnitStride + lane * 4);
+    };
+    auto store_b = [&](UnitRegs& x, int buf) {
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            settle(x.stage[i]);
+            *reinterpret_cast<u32x4*>(tile + buf * kBuf + dst[i]) = x.stage[i];
+        }
+    };
+    auto landed = [&](UnitRegs& x) {
+#pragma unroll
+        for (int r = 0; r < RB; r++) {
+            settle(x.a[r].v[0]);
+            settle(x.a[r].v[1]);
+            settle(x.a[r].idx);
+        }
     };
     auto multiply_from = [&](const AFrag(&a)[RB], int buf) {
 #pragma unroll
@@ -276,44 +331,56 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
         }
     };
 
-    AFrag a0[RB], a1[RB];
+    // Pipeline, per unit u (records two units ahead, the tile one buffer ahead; queue oldest first):
+    //   in flight at the top        records(u), tile(u+1), records(u+1)
+    //   wait until only kLoadsA stay   -> records(u) and tile(u+1) have landed
+    //   tile(u+1) -> the other LDS buffer; issue tile(u+2), records(u+2); multiply unit u; barrier
+    // Loads past the batch's end repeat its last unit, so every path issues the same loads and the
+    // wait count is a constant.  A buffer is written only after the barrier that follows its last reader.
+    UnitRegs x[3];
     int u = u0;  // every wave of the workgroup walks the same units: the barriers below are uniform
     if (u < u1) {
-        fetch_b(u);
-#pragma unroll
-        for (int r = 0; r < RB; r++)
-            a0[r] = load_a(rec[r] + (size_t)u * kRecordBytes, lane);
-        store_b(0);
+        const int last = u1 - 1;
+        auto ahead = [&](int d) { return u + d < last ? u + d : last; };
+        issue_unit(x[0], u);
+        issue_unit(x[1], ahead(1));
+        wait_loads<kLoadsA + CH + kLoadsA>();  // the first tile
+        store_b(x[0], 0);
         __syncthreads();
-        while (true) {
-            // even unit: records in a0, tile in buffer 0
-            bool more = u + 1 < u1;
-            if (more) {
-                fetch_b(u + 1);
-#pragma unroll
-                for (int r = 0; r < RB; r++)
-                    a1[r] = load_a(rec[r] + (size_t)(u + 1) * kRecordBytes, lane);
-            }
-            multiply_from(a0, 0);
-            if (!more)
-                break;
-            store_b(1);  // buffer 1 was last read before the previous barrier
+        auto phase = [&](auto kc) {  // unit u, whose registers are set kc
+            constexpr int k = decltype(kc)::value;
+            const int buf = (u - u0) & 1;
+            wait_loads<kLoadsA>();
+            landed(x[k]);
+            store_b(x[(k + 1) % 3], buf ^ 1);
+            issue_unit(x[(k + 2) % 3], ahead(2));
+            multiply_from(x[k].a, buf);
             __syncthreads();
             ++u;
-            // odd unit: records in a1, tile in buffer 1
-            more = u + 1 < u1;
-            if (more) {
-                fetch_b(u + 1);
+        };
+        // Whole rounds of three units, then the rest: no exit from inside a round, so that every
+        // path through the loop carries the same loads in the same registers.
+        const int units_here = u1 - u0;
+        for (int round = units_here / 3; round > 0; round--) {
+            phase(std::integral_constant<int, 0>{});
+            phase(std::integral_constant<int, 1>{});
+            phase(std::integral_constant<int, 2>{});
+        }
+        const int rest = units_here % 3;
+        if (rest >= 1) {
+            phase(std::integral_constant<int, 0>{});
+            if (rest >= 2)
+                phase(std::integral_constant<int, 1>{});
+        }
+        // the repeated loads of the last phases are still on their way into registers that the
+        // stores below may reuse
+        wait_loads<0>();
 #pragma unroll
-                for (int r = 0; r < RB; r++)
-                    a0[r] = load_a(rec[r] + (size_t)(u + 1) * kRecordBytes, lane);
-            }
-            multiply_from(a1, 1);
-            if (!more)
-                break;
-            store_b(0);
-            __syncthreads();
-            ++u;
+        for (int k = 0; k < 3; k++) {
+            landed(x[k]);
+#pragma unroll
+            for (int i = 0; i < CH; i++)
+                settle(x[k].stage[i]);
         }
     }
 
@@ -354,7 +421,10 @@ int launch_shared_b_nt(hipStream_t s, const void* packed, const void* B, void* o
 #define A24_CASE(RB_, W_)         \
     if (rb == RB_ && waves == W_) \
         return launch_shared_b<NT, RB_, W_>(s, packed, B, out, M, N, K, split_k, ldb, ldo, slab);
-    A24_CASE(2, 4) A24_CASE(2, 8) A24_CASE(4, 2) A24_CASE(4, 4) A24_CASE(4, 8) A24_CASE(8, 2) A24_CASE(8, 4)
+    A24_CASE(2, 4) A24_CASE(2, 8)
+    if constexpr (NT <= 2) {  // three record sets of four row blocks do not fit the registers beside 64 tokens
+        A24_CASE(4, 2) A24_CASE(4, 4) A24_CASE(4, 8)
+    }
 #undef A24_CASE
     return static_cast<int>(hipErrorInvalidValue);
 }
@@ -433,8 +503,11 @@ __global__ __launch_bounds__(256) void a24_split_pack_kernel(const uint16_t* __r
     if (record >= records)
         return;
     const int L = static_cast<int>(id & 63);
-    const long rb = record / units;
-    const int u = static_cast<int>(record - rb * units);
+    // records are numbered ((rb / 8) * units + u) * 8 + rb % 8
+    const long group = record / (static_cast<long>(units) * kGroupBlocks);
+    const int within = static_cast<int>(record - group * units * kGroupBlocks);
+    const int u = within / kGroupBlocks;
+    const long rb = group * kGroupBlocks + within % kGroupBlocks;
     const size_t row = (size_t)(rb * 16 + (L & 15)) * K + (size_t)u * 128 + (L >> 4) * 8;
     uint8_t* rec = packed + (size_t)record * kRecordBytes;
     typedef unsigned short u16x8 __attribute__((ext_vector_type(8)));

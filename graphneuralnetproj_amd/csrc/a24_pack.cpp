@@ -68,7 +68,7 @@ int pack(const uint16_t* A1, int M, int K, uint8_t* packed)
 {
     if (!A1 || !packed)
         return kErrNullPointer;
-    if (M <= 0 || K <= 0 || M % kRows != 0 || K % kUnitCols != 0)
+    if (M <= 0 || K <= 0 || M % (kRows * kGroupBlocks) != 0 || K % kUnitCols != 0)
         return kErrBadShape;
     const int units = K / kUnitCols;
     const long blocks = M / kRows;
@@ -77,7 +77,7 @@ int pack(const uint16_t* A1, int M, int K, uint8_t* packed)
     parallel_for(blocks, [=](long b0, long b1) {
         for (long rb = b0; rb < b1; rb++) {
             for (int u = 0; u < units; u++) {
-                uint8_t* rec = packed + (rb * units + u) * kRecordBytes;
+                uint8_t* rec = packed + record_index(rb, u, units) * kRecordBytes;
                 for (int L = 0; L < 64; L++) {
                     const uint16_t* row = A1 + (rb * kRows + L % 16) * static_cast<long>(K) + static_cast<long>(u) * kUnitCols;
                     uint32_t word = 0;

@@ -384,7 +384,7 @@ extern "C" int HeteroSparse_Decompose(const uint16_t* A_h, uint16_t* A1_h, uint1
 
 extern "C" long HeteroSparse_PackedBytes(int M, int K)
 {
-    if (M <= 0 || K <= 0 || M % a24::kRows != 0 || K % a24::kUnitCols != 0)
+    if (M <= 0 || K <= 0 || M % (a24::kRows * a24::kGroupBlocks) != 0 || K % a24::kUnitCols != 0)
         return a24::kErrBadShape;
     return a24::bytes(M, K);
 }
@@ -396,8 +396,8 @@ extern "C" int HeteroSparse_PackA1(const uint16_t* A1_h, int M, int K, void* Pac
 
 extern "C" int HeteroSparse_DeviceSplitPack(void* stream, const void* A_d, int M, int K, void* Packed_A1_d, void* A2_d)
 {
-    if (!A_d || !Packed_A1_d || M <= 0 || K <= 0 || M % a24::kRows != 0 || K % a24::kUnitCols != 0) {
-        std::fprintf(stderr, "HeteroSparse_DeviceSplitPack: need M %% 16 == 0, K %% 128 == 0 and non-null pointers (M=%d K=%d)\n", M, K);
+    if (!A_d || !Packed_A1_d || M <= 0 || K <= 0 || M % (a24::kRows * a24::kGroupBlocks) != 0 || K % a24::kUnitCols != 0) {
+        std::fprintf(stderr, "HeteroSparse_DeviceSplitPack: need M %% 128 == 0, K %% 128 == 0 and non-null pointers (M=%d K=%d)\n", M, K);
         return tcsl_error_invalid_value();
     }
     return a24_launch_split_pack(stream, A_d, Packed_A1_d, A2_d, M, K);
@@ -413,14 +413,16 @@ struct A24Plan {
 
 A24Plan a24_default_plan(int M, int N, int K)
 {
-    // From a sweep on the OPT-30B shapes: workgroups of four waves with two row blocks each (128
-    // rows) that share the activation tile through LDS are the best or within 4 % of it for every
-    // token count, and split-K until about two workgroups per compute unit exist.
-    A24Plan p{2, 4, 1, 1};
+    // From sweeps on the OPT-30B shapes: waves that own two row blocks each and share the activation
+    // tile through LDS; sixteen of them per workgroup where the rows allow (256 rows, two groups of
+    // records: best for every token count), else eight (one group); split-K until about one
+    // sixteen-wave workgroup per compute unit exists.
+    A24Plan p{2, M % 256 == 0 ? 8 : 4, 1, 1};
     (void)N;
     const long groups = M / (16 * p.row_blocks * p.waves);
+    const long target = 1792 / p.waves;
     const int units = K / a24::kUnitCols;
-    while (groups * p.split_k < 448) {
+    while (groups * p.split_k < target) {
         const int s2 = p.split_k * 2;
         const int per = (units + s2 - 1) / s2;
         if (per < 2 || static_cast<long>(per) * (s2 - 1) >= units)
@@ -444,6 +446,8 @@ bool a24_shape_ok(int M, int N, int K, int split_k, int row_blocks, int waves, i
         return false;
     if (share_b) {  // the kernel table of this layout, and whole workgroups only
         if (row_blocks < 2 || waves < 2 || row_blocks * waves < 8 || M % (16 * row_blocks * waves) != 0)
+            return false;
+        if (row_blocks > (N == 64 ? 2 : 4))  // three sets of record registers: what fits beside the accumulators
             return false;
         return true;
     }

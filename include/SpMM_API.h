@@ -249,7 +249,8 @@ SPMM_EXPORT int SpMM_CalibrationCopy(void* stream, void* dst, const void* src, l
  * (build/SpMM_API.cuh:40-52), with A2 going to a second kernel on another stream
  * (kernel_benchmark/spmm_test.cu:285-330,462-560).  Here A1 is stored as records in the operand
  * order of gfx950's v_smfmac_f32_16x16x32_f16 (16 rows x 128 columns, 2304 bytes: 2048 bytes of
- * fp16 values, 256 bytes of 2-bit positions; 1.125 bytes per dense element at any sparsity).
+ * fp16 values, 256 bytes of 2-bit positions; 1.125 bytes per dense element at any sparsity), the
+ * records of eight consecutive 16-row blocks stored together unit by unit.
  */
 
 /*
@@ -264,7 +265,7 @@ SPMM_EXPORT int HeteroSparse_Decompose(const uint16_t* A_h, uint16_t* A1_h, uint
 /*
  * Stand in for InitSparseMatrixA1_Vec_Sparse_Load and inspect_metadata (csrc/SpMM_API.cu:1127-1553),
  * which produce mma.sp's value and metadata arrays; the bytes differ by design (other hardware).
- * HeteroSparse_PackedBytes: size of the records of an M x K matrix (M % 16 == 0, K % 128 == 0), or -1.
+ * HeteroSparse_PackedBytes: size of the records of an M x K matrix (M % 128 == 0, K % 128 == 0), or -1.
  * HeteroSparse_PackA1: fills Packed_h (host memory of that size) from row-major A1_h.  Returns 0,
  * -1 bad shape, -3 null pointer, -6 if some group of four holds more than two kept values.
  */
@@ -273,7 +274,7 @@ SPMM_EXPORT int HeteroSparse_PackA1(const uint16_t* A1_h, int M, int K, void* Pa
 
 /*
  * Split and pack on the GPU, for a weight that is already in device memory (row-major M x K fp16 at
- * A_d, M % 16 == 0, K % 128 == 0): Packed_A1_d receives the records (HeteroSparse_PackedBytes bytes),
+ * A_d, M % 128 == 0, K % 128 == 0): Packed_A1_d receives the records (HeteroSparse_PackedBytes bytes),
  * A2_d, if not NULL, the dense residual (M*K fp16, zero where nothing is left), ready for
  * SpMM_DeviceEncodeOffsets / SpMM_DeviceEncodeItems.  Same bits as HeteroSparse_Decompose followed by
  * HeteroSparse_PackA1.  Only enqueues a kernel on `stream`; returns a hipError_t value.  The reference

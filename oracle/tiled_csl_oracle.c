@@ -479,8 +479,9 @@ void oracle_decompose(const uint16_t *A, uint16_t *A1, uint16_t *A2, long length
  * group g = L / 16), step s in 0..3 and slot j in 0..3, the fp16 value at byte
  * (s / 2) * 1024 + L * 16 + ((s % 2) * 4 + j) * 2 belongs to column
  * s * 32 + g * 8 + (j / 2) * 4 + q of the record, where q is the 2-bit field at bit
- * 8 * s + 2 * j of the 32-bit word at byte 2048 + L * 4.  Records are ordered by
- * 16-row block, then by 128-column unit.  Returns 0, or -1 if two slots of one group
+ * 8 * s + 2 * j of the 32-bit word at byte 2048 + L * 4.  Records are ordered by group
+ * of eight 16-row blocks, then by 128-column unit, then by block within the group:
+ * block rb, unit u is record ((rb / 8) * (K / 128) + u) * 8 + rb % 8 (M % 128 == 0).  Returns 0, or -1 if two slots of one group
  * of four name the same column or come in descending order.
  */
 int oracle_a24_unpack(const uint8_t *packed, int M, int K, uint16_t *A_out)
@@ -489,7 +490,7 @@ int oracle_a24_unpack(const uint8_t *packed, int M, int K, uint16_t *A_out)
     memset(A_out, 0, sizeof(uint16_t) * (size_t)M * (size_t)K);
     for (int rb = 0; rb < M / 16; rb++) {
         for (int u = 0; u < units; u++) {
-            const uint8_t *rec = packed + ((size_t)rb * units + u) * 2304;
+            const uint8_t *rec = packed + (((size_t)(rb / 8) * units + u) * 8 + (size_t)(rb % 8)) * 2304;
             for (int L = 0; L < 64; L++) {
                 uint32_t word;
                 memcpy(&word, rec + 2048 + L * 4, 4);

@@ -103,8 +103,10 @@ def test_decompose_rejects_bad_length(spmm):
 
 
 def test_oracle_unpack_reads_a_hand_built_record(oracle):
-    """One 16 x 128 record written byte by byte from the layout's definition."""
-    M, K = 16, 128
+    """One 16 x 128 record written byte by byte from the layout's definition, as record 3 of the
+    eight that a 128 x 128 matrix has (row block 3); the others hold zeros at valid positions."""
+    M, K = 128, 128
+    BLOCK = 3
     rec = np.zeros(2304, dtype=np.uint8)
     words = np.zeros(64, dtype=np.uint32)
     for L in range(64):  # every group of four: positions (0, 1), zero values
@@ -121,23 +123,26 @@ def test_oracle_unpack_reads_a_hand_built_record(oracle):
             words[L] = (int(words[L]) & ~(3 << shift)) | (q_pair[t] << shift)
         off = (s // 2) * 1024 + L * 16 + ((s % 2) * 4 + j) * 2
         rec[off:off + 2] = np.array([value], dtype=H).view(np.uint8)
-        expect[L % 16, s * 32 + (L // 16) * 8 + (j // 2) * 4 + q_pair[j % 2]] = value
+        expect[BLOCK * 16 + L % 16, s * 32 + (L // 16) * 8 + (j // 2) * 4 + q_pair[j % 2]] = value
 
     put(0, 0, 0, (0, 1), 1.5)      # row 0, column 0
     put(0, 0, 3, (1, 3), -2.0)     # row 0, second group of the lane: column 4 + 3
     put(17, 2, 1, (2, 3), 3.0)     # row 1, column 2*32 + 1*8 + 3
     put(63, 3, 2, (1, 2), 0.25)    # row 15, column 3*32 + 3*8 + 4 + 1
     rec[2048:] = words.view(np.uint8)
-    got = oracle.a24_unpack(rec, M, K)
+    empty = np.zeros(2304, dtype=np.uint8)
+    empty[2048:] = np.full(64, 0x44444444, dtype=np.uint32).view(np.uint8)  # positions (0, 1) everywhere
+    packed = np.concatenate([rec if b == BLOCK else empty for b in range(8)])
+    got = oracle.a24_unpack(packed, M, K)
     assert np.array_equal(got.view(np.uint16), expect.view(np.uint16))
-    assert got[0, 0] == H(1.5) and got[0, 7] == H(-2.0) and got[1, 75] == H(3.0) and got[15, 125] == H(0.25)
+    assert got[48, 0] == H(1.5) and got[48, 7] == H(-2.0) and got[49, 75] == H(3.0) and got[63, 125] == H(0.25)
     words[5] = 0  # positions (0, 0) in every pair: not a valid record
     rec[2048:] = words.view(np.uint8)
     with pytest.raises(ValueError):
-        oracle.a24_unpack(rec, M, K)
+        oracle.a24_unpack(np.concatenate([rec if b == BLOCK else empty for b in range(8)]), M, K)
 
 
-@pytest.mark.parametrize("M,K,keep", [(16, 128, 0.5), (128, 256, 0.2), (256, 1024, 0.8), (128, 128, 0.0)])
+@pytest.mark.parametrize("M,K,keep", [(128, 128, 0.5), (128, 256, 0.2), (384, 1024, 0.8), (128, 128, 0.0)])
 def test_pack_round_trip(spmm, oracle, M, K, keep):
     rng = np.random.default_rng(M + K)
     A1, _ = oracle.decompose(_rand_sparse(rng, M, K, keep))
@@ -148,15 +153,15 @@ def test_pack_round_trip(spmm, oracle, M, K, keep):
 
 
 def test_pack_rejects_three_of_four_and_bad_shapes(spmm):
-    A = np.zeros((16, 128), dtype=H)
+    A = np.zeros((128, 128), dtype=H)
     A[3, 8:11] = 1
     with pytest.raises(spmm.SpMMError) as e:
         spmm.HeteroSparse_PackA1(A)
     assert e.value.code == -6
     with pytest.raises(spmm.SpMMError):
-        spmm.HeteroSparse_PackA1(np.zeros((16, 64), dtype=H))
+        spmm.HeteroSparse_PackA1(np.zeros((128, 64), dtype=H))
     with pytest.raises(spmm.SpMMError):
-        spmm.HeteroSparse_PackA1(np.zeros((8, 128), dtype=H))
+        spmm.HeteroSparse_PackA1(np.zeros((64, 128), dtype=H))
 
 
 def test_suggested_split_leaves_no_batch_empty(spmm):
@@ -166,3 +171,21 @@ def test_suggested_split_leaves_no_batch_empty(spmm):
             units = K // 128
             per = -(-units // s)
             assert s >= 1 and per * (s - 1) < units
+
+
+def test_record_order_groups_eight_row_blocks(spmm, oracle):
+    """Record of row block rb and unit u sits at ((rb // 8) * units + u) * 8 + rb % 8: a matrix with one
+    value per (row block, unit) cell, whose value names the cell, must show each value in that record."""
+    M, K = 384, 512
+    units = K // 128
+    A = np.zeros((M, K), dtype=H)
+    for rb in range(M // 16):
+        for u in range(units):
+            A[rb * 16, u * 128] = H(rb * units + u + 1)  # lane 0, step 0, slot 0 of the record
+    packed = spmm.HeteroSparse_PackA1(A).reshape(-1, 2304)
+    assert packed.shape[0] == (M // 16) * units
+    first = packed[:, :2].copy().view(H).reshape(-1)   # lane 0's first value of every record
+    for rb in range(M // 16):
+        for u in range(units):
+            assert first[((rb // 8) * units + u) * 8 + rb % 8] == H(rb * units + u + 1)
+    assert np.array_equal(oracle.a24_unpack(packed.reshape(-1), M, K).view(np.uint16), A.view(np.uint16))
