@@ -160,3 +160,13 @@ def test_built_kernels_pass():
     r = subprocess.run([sys.executable, CHECKER, asm, "tcsl_spmm_kernel"], capture_output=True, text=True)
     assert r.returncode == 0, r.stdout
     assert r.stdout.count("ok ") >= 10
+
+
+def test_built_sparse_mfma_kernels_pass():
+    """The 2:4 kernel that issues its loads from inline assembly: every instantiation in the launch table."""
+    asm = os.path.join(HERE, "..", "graphneuralnetproj_amd", "csrc", "obj", "a24_kernels.gfx950.s")
+    if not os.path.exists(asm):
+        pytest.skip("library not built in this tree")
+    r = subprocess.run([sys.executable, CHECKER, asm, "a24_spmm_shared_b_kernel"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout
+    assert r.stdout.count("ok ") == 12  # 2 + 5 + 5 launch shapes for 64, 32 and up to 16 tokens
