@@ -413,21 +413,30 @@ struct A24Plan {
 
 A24Plan a24_default_plan(int M, int N, int K)
 {
-    // From sweeps on the OPT-30B shapes: waves that own two row blocks each and share the activation
-    // tile through LDS; sixteen of them per workgroup where the rows allow (256 rows, two groups of
-    // records: best for every token count), else eight (one group); split-K until about one
-    // sixteen-wave workgroup per compute unit exists.
+    // From sweeps over the OPT-30B and OPT-66B shapes (N = 16 and 64): waves that own two row blocks
+    // each and share the activation tile through LDS, eight of them per workgroup where the rows
+    // allow (256 rows, two groups of records), else four; and the split-K with the least estimated
+    // time: rounds of up to 256 workgroups, each round streaming its share of the records at one
+    // compute unit's rate plus a fixed cost, and a small cost per slab.  That picks the counts the
+    // sweeps found fastest: just under 256 workgroups (216 to 252) where the rows allow, else e.g.
+    // 432 rather than 144 or 288.
     A24Plan p{2, M % 256 == 0 ? 8 : 4, 1, 1};
     (void)N;
     const long groups = M / (16 * p.row_blocks * p.waves);
-    const long target = 1792 / p.waves;
     const int units = K / a24::kUnitCols;
-    while (groups * p.split_k < target) {
-        const int s2 = p.split_k * 2;
-        const int per = (units + s2 - 1) / s2;
-        if (per < 2 || static_cast<long>(per) * (s2 - 1) >= units)
-            break;
-        p.split_k = s2;
+    const double bytes = static_cast<double>(a24::bytes(M, K));
+    constexpr double kUnitBytesPerUs = 25.4e3, kRoundUs = 6.0, kSlabUs = 0.5;
+    double best = 0.0;
+    for (int s = 1; s <= 32 && s <= units; s++) {
+        const int per = (units + s - 1) / s;
+        if ((s > 1 && per < 2) || static_cast<long>(per) * (s - 1) >= units)
+            continue;  // batches of one unit, or an empty last batch
+        const long n = groups * s;
+        const double cost = static_cast<double>((n + 255) / 256) * (bytes / n / kUnitBytesPerUs + kRoundUs) + kSlabUs * s;
+        if (best == 0.0 || cost < best * 0.999) {
+            best = cost;
+            p.split_k = s;
+        }
     }
     return p;
 }
