@@ -8,7 +8,8 @@ figures are printed per token count, in microseconds per call (events around `--
 weights rotated over several copies so that no cache level holds the stream):
   csl     SpMM_SplitK_API on the whole matrix with the planner's Split_K;
   a1      the 2:4 kernel alone (its bytes do not depend on the sparsity);
-  hybrid  HeteroSparse_SpMM_API: 2:4 kernel, the residual's Tiled-CSL kernel, one reduction;
+  hybrid  HeteroSparse_SpMM_API: 2:4 kernel, then the residual's Tiled-CSL kernel (--residual-split-k), which
+          adds all slabs up itself where its launch allows, else one reduction kernel;
   2-str   the same with HETERO_FLAG_TWO_STREAMS (the two kernels side by side).
 """
 import argparse
@@ -28,6 +29,8 @@ def main():
     ap.add_argument("--n", default="8,16,32,64")
     ap.add_argument("--iters", type=int, default=200)
     ap.add_argument("--copies", type=int, default=3)
+    ap.add_argument("--residual-split-k", type=int, default=0,
+                    help="Split_K of the residual's Tiled-CSL kernel (0 = the planner's choice for the whole matrix)")
     args = ap.parse_args()
     G.load_library()
     M, K = args.m, args.k
@@ -77,11 +80,12 @@ def main():
                 first = False
             t_csl = time_us(lambda i: G.SpMM_SplitK_API(st, None, d_items[i % c], d_offs[i % c], B, C, M, N, K, W, s0))
             t_a1 = time_us(lambda i: G.HeteroSparse_A1_Partials(st, d_p[i % c], B, W, M, N, K, s1))
-            t_h = time_us(lambda i: G.HeteroSparse_SpMM_API(st, d_p[i % c], d_i2[i % c], d_o2[i % c], B, C, M, N, K, W, s1, s0))
-            t_2 = time_us(lambda i: G.HeteroSparse_SpMM_API(st, d_p[i % c], d_i2[i % c], d_o2[i % c], B, C, M, N, K, W, s1, s0,
+            S2 = args.residual_split_k or s0
+            t_h = time_us(lambda i: G.HeteroSparse_SpMM_API(st, d_p[i % c], d_i2[i % c], d_o2[i % c], B, C, M, N, K, W, s1, S2))
+            t_2 = time_us(lambda i: G.HeteroSparse_SpMM_API(st, d_p[i % c], d_i2[i % c], d_o2[i % c], B, C, M, N, K, W, s1, S2,
                                                            G.HETERO_FLAG_TWO_STREAMS))
             print(f"sparsity {sp} N={N:2d}: csl {t_csl:6.1f} us (Split_K {s0}) | a1 {t_a1:6.1f} us (Split_K {s1}, "
-                  f"{packed.nbytes / t_a1 / 1e6:.2f} TB/s) | hybrid {t_h:6.1f} us | 2-str {t_2:6.1f} us", flush=True)
+                  f"{packed.nbytes / t_a1 / 1e6:.2f} TB/s) | hybrid {t_h:6.1f} us (residual Split_K {S2}) | 2-str {t_2:6.1f} us", flush=True)
         del d_items, d_offs, d_p, d_i2, d_o2
         torch.cuda.empty_cache()
 
