@@ -308,10 +308,14 @@ SPMM_EXPORT int HeteroSparse_SuggestSplitK(int M_Global, int N_Global, int K_Glo
 
 /*
  * The 2:4 kernel alone: batch b of ceil((K/128)/Split_K) units writes fp16 A1*B partial sums to
- * Partials[b*M*N ..).  RowBlocks (16-row blocks per workgroup: 1, 2, 4, 8) and Waves (waves per
- * workgroup: 1, 2, 4, 8) choose the launch shape; 0, 0 = the library's choice.  ShareB = 0: the
- * waves of a workgroup split the batch's columns and add their sums up; ShareB = 1: they own
- * RowBlocks row blocks each and share the activation tile through LDS (M % (16*RowBlocks*Waves) == 0).  hipErrorInvalidValue for shapes the kernel table does not hold.  For tuning and tests.
+ * Partials[b*M*N ..).  RowBlocks, Waves and ShareB choose the launch shape; 0, 0 = the library's
+ * choice (ShareB is then ignored).
+ *   ShareB = 1  each of the Waves (2, 4, 8) waves of a workgroup owns RowBlocks (2 or 4; 2 for N = 64)
+ *               16-row blocks and all share the activation tile through LDS; RowBlocks * Waves >= 8 and
+ *               M % (16 * RowBlocks * Waves) == 0.  The library's own launches are of this kind.
+ *   ShareB = 0  a workgroup owns RowBlocks (1, 2, 4, 8) blocks; its Waves (1, 2, 4, 8) waves split the
+ *               batch's columns and add their sums up.
+ * hipErrorInvalidValue for shapes the kernel tables do not hold.  For tuning and tests.
  */
 SPMM_EXPORT int HeteroSparse_A1_Partials(void* stream, const void* Packed_A1, const void* B, void* Partials, int M_Global,
                                          int N_Global, int K_Global, int Split_K, int RowBlocks, int Waves, int ShareB);
