@@ -600,7 +600,15 @@ extern "C" int a24_side_begin(void* stream, void** side)
         for (int i = 0; i < side_used && !e; i++)
             if (side_table[i].owner == s)
                 e = &side_table[i];
-        if (!e && side_used < 32) {
+        // Streams and events are not created while the caller's stream is being captured into a
+        // graph (not a call a capture allows): such a call runs on the caller's stream alone unless
+        // an earlier, eager call has already made the pair.
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (!e && hipStreamIsCapturing(s, &capturing) != hipSuccess) {
+            (void)hipGetLastError();
+            capturing = hipStreamCaptureStatusActive;
+        }
+        if (!e && side_used < 32 && capturing == hipStreamCaptureStatusNone) {
             SideStream n{s, nullptr, nullptr, nullptr};
             if (hipStreamCreateWithFlags(&n.side, hipStreamNonBlocking) != hipSuccess
                 || hipEventCreateWithFlags(&n.fork, hipEventDisableTiming) != hipSuccess

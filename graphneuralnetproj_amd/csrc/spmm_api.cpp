@@ -9,6 +9,7 @@
 
 #include "../../include/SpMM_API.h"
 #include "a24_format.h"
+#include "counter_pages.h"
 #include "launch_plan.h"
 #include "tiled_csl_format.h"
 
@@ -25,6 +26,8 @@ int a24_launch_spmm(void* stream, const void* packed, const void* B, void* out, 
 int a24_launch_split_pack(void* stream, const void* A, void* packed, void* residual, int M, int K);
 int a24_side_begin(void* stream, void** side);
 int a24_side_end(void* stream, void* side);
+int tcsl_stream_capture(void* stream, unsigned long long* id);
+int tcsl_stream_idle(void* stream);
 void* tcsl_event_create(void);
 void tcsl_event_destroy(void* e);
 int tcsl_event_record(void* e, void* stream);
@@ -103,24 +106,22 @@ tcsl::LaunchPlan cached_plan(int M, int N, int K, int Split_K, bool row_major)
     return p;
 }
 
-// The fused split-K reduction counts arrivals in one of 64 pages of device counters.  Calls on
-// one stream run in order and can share a page; calls on different streams may overlap, so each
-// stream gets a page of its own, first come first served.  -1 when all pages are taken (the call
-// then uses the separate reduction kernel).
+// The fused split-K reduction counts arrivals in a page of device counters that no launch
+// which might overlap this one may use (counter_pages.h has the rules).  -1 when no page can be
+// had: the call then runs the reduction as a second kernel.  The caller holds pages.mutex().
+tcsl::CounterPages& counter_pages()
+{
+    static tcsl::CounterPages pages;
+    return pages;
+}
+
 int counter_page(void* stream)
 {
-    constexpr int kPages = 64;
-    static std::mutex mu;
-    static void* owner[kPages];
-    static int used = 0;
-    std::lock_guard<std::mutex> lock(mu);
-    for (int i = 0; i < used; i++)
-        if (owner[i] == stream)
-            return i;
-    if (used == kPages)
+    unsigned long long capture_id = 0;
+    const int capturing = tcsl_stream_capture(stream, &capture_id);
+    if (capturing < 0)
         return -1;
-    owner[used] = stream;
-    return used++;
+    return counter_pages().acquire(stream, capturing == 1, capture_id, [](void* s) { return tcsl_stream_idle(s) == 1; });
 }
 
 // What varies between the entry points that end in the same two launches.
@@ -147,8 +148,13 @@ int launch_main(void* stream, const void* Compressed_A, const int* TileOffsets, 
     // Only the layout whose workgroup owns a single tile row fuses the reduction: its last arriver
     // adds up 128 rows.  In the row-sharing layout one workgroup would be left with W x 128 rows of
     // every slab while the rest of the chip idles, which measured slower than the second kernel.
-    if (fused_out && p.mode == 1 && M / tcsl::kTileRows <= 4096)
+    // A page from the pool stays this call's until the launch is enqueued (the lock): from then
+    // on its stream counts as busy and the page cannot change hands.
+    std::unique_lock<std::mutex> page_lock;
+    if (fused_out && p.mode == 1 && M / tcsl::kTileRows <= 4096) {
+        page_lock = std::unique_lock<std::mutex>(counter_pages().mutex());
         page = counter_page(stream);
+    }
     if (fused)
         *fused = page >= 0;
     // The plan's wave count is tuned on 80 % sparse weights.  Sparser ones want every wave the
@@ -170,6 +176,8 @@ int launch_main(void* stream, const void* Compressed_A, const int* TileOffsets, 
                             page >= 0 ? fused_out : nullptr, static_cast<int>(ldc), page, dense_waves);
 }
 
+int check_call(const void* Compressed_A, const int* TileOffsets, const void* B, const void* C, int M, int N, int K,
+               bool have_workspace, int Split_K);
 int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* C, int M, int N,
                 int K, void* Reduction_Workspace, int Split_K, const CallOptions& o);
 }  // namespace
@@ -292,8 +300,9 @@ extern "C" float SpMM_EventElapsedMs(void* start, void* stop)
 
 namespace {
 
-int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* C, int M, int N,
-                int K, void* Reduction_Workspace, int Split_K, const CallOptions& o)
+// The checks every product entry point makes before anything is launched; 0 = fine.
+int check_call(const void* Compressed_A, const int* TileOffsets, const void* B, const void* C, int M, int N, int K,
+               bool have_workspace, int Split_K)
 {
     if (N != 8 && N != 16 && N != 32 && N != 64) {
         std::printf("MM_Sparse_API Error: Unsupported N dimension %d!\n", N);
@@ -304,7 +313,7 @@ int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, 
                      M, K, Split_K);
         return tcsl_error_invalid_value();
     }
-    if (!Compressed_A || !TileOffsets || !B || !C || (Split_K > 1 && !Reduction_Workspace)) {
+    if (!Compressed_A || !TileOffsets || !B || !C || (Split_K > 1 && !have_workspace)) {
         std::fprintf(stderr, "SpMM_SplitK_API: null device pointer\n");
         return tcsl_error_invalid_value();
     }
@@ -313,6 +322,14 @@ int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, 
         std::fprintf(stderr, "SpMM_SplitK_API: Split_K=%d too large for M=%d\n", Split_K, M);
         return tcsl_error_invalid_value();
     }
+    return 0;
+}
+
+int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B, void* C, int M, int N,
+                int K, void* Reduction_Workspace, int Split_K, const CallOptions& o)
+{
+    if (const int bad = check_call(Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace != nullptr, Split_K))
+        return bad;
     const int ldb = o.ldb ? static_cast<int>(o.ldb) : K;
     const long ldc = o.ldc ? o.ldc : M;
     // optional events bracket the main kernel only (not the reduction)
@@ -531,13 +548,15 @@ extern "C" int HeteroSparse_SpMM_API(void* stream, const void* Packed_A1, const 
             return rc;
         CallOptions o;
         o.separate_reduction = true;
-        if ((rc = launch_main(side, Compressed_A2, TileOffsets_A2, B, ws, M, N, K, Split_K_A2, o, K, M, false, nullptr, 0,
-                              nullptr)) != 0)
-            return rc;
-        if ((rc = a24_launch_spmm(stream, Packed_A1, B, ws_a1, M, N, K, Split_K_A1, d.row_blocks, d.waves, d.share_b, K, M,
-                                  mn)) != 0)
-            return rc;
-        if ((rc = a24_side_end(stream, side)) != 0)
+        rc = launch_main(side, Compressed_A2, TileOffsets_A2, B, ws, M, N, K, Split_K_A2, o, K, M, false, nullptr, 0,
+                         nullptr);
+        if (rc == 0)
+            rc = a24_launch_spmm(stream, Packed_A1, B, ws_a1, M, N, K, Split_K_A1, d.row_blocks, d.waves, d.share_b, K, M,
+                                 mn);
+        // the side stream joins the caller's whatever happened in between: a fork left open would
+        // leave the two streams unordered (and invalidate a graph capture that includes this call)
+        const int joined = a24_side_end(stream, side);
+        if (rc != 0 || (rc = joined) != 0)
             return rc;
     } else {
         // One stream: the 2:4 kernel first; the residual's kernel then adds everything up itself where

@@ -59,6 +59,7 @@
 #include <stdint.h>
 
 #include <atomic>
+#include <mutex>
 #include <utility>
 
 namespace {
@@ -94,12 +95,13 @@ constexpr unsigned kMaxLdsBytes = 160 * 1024;  // LDS of one gfx950 compute unit
 constexpr int kDenseTileVectors = 340;         // average vectors per tile from which a unit counts as dense (about 83 % sparsity)
 constexpr int kSparseWaves = 6;                // waves that work on a sparse unit when the launch shape is adaptive
 
-// Arrival counters of the fused split-K reduction: one page per caller stream, one counter per
-// group of output rows.  Zero when the module is loaded; the workgroup that brings a counter to
-// Split_K sets it back to zero, so every call finds them at zero.
-constexpr int kCounterPages = 64;
+// Arrival counters of the fused split-K reduction: pages of one counter per group of output
+// rows, handed out by the host (one page per caller stream, or per graph capture and stream).
+// Zero when the module is loaded; the workgroup that brings a counter to Split_K sets it back to
+// zero, so every call finds them at zero.  Kernels receive a page's address as an argument.
+constexpr int kCounterPages = 256;
 constexpr int kCountersPerPage = 4096;
-__device__ unsigned int tcsl_arrivals[kCounterPages][kCountersPerPage];
+static __device__ __align__(256) unsigned int tcsl_arrivals[kCounterPages][kCountersPerPage];
 
 template<int... Is, typename F>
 __device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F&& f)
@@ -284,9 +286,10 @@ __device__ __forceinline__ void fused_reduction_tail(const _Float16* __restrict_
 
 // ldb = elements between two tokens' vectors in B, ldo = the same for the output (column-major
 // only; the slabs of partial sums use M); relu != 0 clamps the output at zero (final results only).
-// fuse_page >= 0 (Split_K > 1, column-major): `out` receives the slabs of partial sums as usual,
+// arrivals != nullptr (Split_K > 1, column-major): `out` receives the slabs of partial sums as usual,
 // and the last workgroup to finish a group of rows adds the slabs up into fused_out (token stride
-// ldc, clamped if relu) itself; arrivals are counted in tcsl_arrivals[fuse_page].
+// ldc, clamped if relu) itself; arrivals are counted in arrivals[blockIdx.x] (device memory, zero
+// before the launch and after it).
 // blockDim.x = W * 64, grid = (groups of tile rows, Split_K).  Wave w of workgroup (g, b) owns
 // tile row g * W + w of batch b; with KSPLIT the workgroup owns tile row g and its waves share
 // the batch.  avg = tiles per batch = ceil((K / 64) / Split_K).  NB = number of 16-token column blocks;
@@ -301,8 +304,9 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
                                                                 const _Float16* __restrict__ B,
                                                                 _Float16* __restrict__ out, int K, int avg,
                                                                 int wave_counts, int ldb, int M, int ldo,
-                                                                _Float16* __restrict__ fused_out, int ldc,
-                                                                int fuse_page, int relu, int split_k)
+                                                                _Float16* __restrict__ fused_out,
+                                                                unsigned int* __restrict__ arrivals, int ldc,
+                                                                int relu, int split_k)
 {
     // (Argument order: the first 14 dwords are preloaded into scalar registers when a wave starts
     // (-amdgpu-kernarg-preload-count); they are what the way to the first tile's loads needs.
@@ -384,7 +388,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         clear_tile(tile, lane);
         cleared = true;
         // (the arguments that are not preloaded are fetched while the offsets are on their way)
-        asm volatile("" ::"s"(relu), "s"(fuse_page), "s"(ldc), "s"(split_k), "s"(fused_out));
+        asm volatile("" ::"s"(relu), "s"(arrivals), "s"(ldc), "s"(split_k), "s"(fused_out));
         wait_loads<0>();
         settle(wd);
         settle(wreg);
@@ -426,9 +430,9 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         clear_tile(tile, lane);
     if (BLDS)
         __syncthreads();  // the only barrier: every wave of the workgroup reaches it
-    if (!KSPLIT && !active && fuse_page < 0)
+    if (!KSPLIT && !active && !arrivals)
         return;  // (with the fused reduction every wave has to reach the barriers at the end)
-    const bool clamp = relu && fuse_page < 0;  // partial sums are never clamped
+    const bool clamp = relu && !arrivals;  // partial sums are never clamped
 
     auto tile_range = [&](int i, int& begin, int& end) {  // 0 <= i < ntile
         if (i + 1 - wbase >= kWave) {  // slide the window (more than 63 tiles per wave only)
@@ -786,7 +790,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
                         oslab[(r * 16 + q * 4 + i) * NTOK + c * 16 + l15] = h[i];
                 } else {  // the four q-lanes of a token cover 32 bytes
                     _Float16* dst = oslab + (size_t)(c * 16 + l15) * ldo + r * 16 + q * 4;
-                    if (fuse_page >= 0)
+                    if (arrivals)
                         store_through(dst, h);
                     else
                         *reinterpret_cast<half4*>(dst) = h;
@@ -842,7 +846,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
             const int tok = e >> 4, part = e & 15;
             const half8 v = *reinterpret_cast<const half8*>(tile + tok * kTokStride + part * 16);
             _Float16* dst = oslab + (size_t)(c * 16 + tok) * ldo + part * 8;
-            if (fuse_page >= 0)
+            if (arrivals)
                 store_through(dst, v);
             else
                 *reinterpret_cast<half8*>(dst) = v;
@@ -851,12 +855,12 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
     };
     if (KSPLIT || active)
         write_out();
-    if (ROWMAJ || fuse_page < 0)
+    if (ROWMAJ || !arrivals)
         return;
 
     const int row0 = (KSPLIT ? blockIdx.x : blockIdx.x * W) * kTileRows;
     fused_reduction_tail(out, fused_out, M, NTOK, ldc, split_k, relu, row0, (KSPLIT ? 1 : W) * kTileRows,
-                         &tcsl_arrivals[fuse_page][blockIdx.x], reinterpret_cast<unsigned int*>(lds),
+                         arrivals + blockIdx.x, reinterpret_cast<unsigned int*>(lds),
                          W * kWave);
 }
 
@@ -906,10 +910,44 @@ __global__ __launch_bounds__(256) void tcsl_copy_kernel(u32x4* __restrict__ dst,
         dst[i] = src[i];
 }
 
+// Device address of the counter pages on the current device.  A __device__ array's name in
+// host code is a handle, not an address, and every device holds its own copy: the address is
+// asked for once per device (with that device current) and kept.
+struct DeviceArrays {
+    unsigned int* arrivals;      // tcsl_arrivals
+};
+constexpr int kMaxDevices = 64;
+int device_arrays(DeviceArrays* out)
+{
+    static std::mutex mu;
+    static DeviceArrays table[kMaxDevices];
+    static std::atomic<bool> known[kMaxDevices];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess)
+        return static_cast<int>(e);
+    if (dev < 0 || dev >= kMaxDevices)
+        return static_cast<int>(hipErrorInvalidDevice);
+    if (!known[dev].load(std::memory_order_acquire)) {
+        std::lock_guard<std::mutex> lock(mu);
+        if (!known[dev].load(std::memory_order_relaxed)) {
+            DeviceArrays a{nullptr};
+            if ((e = hipGetSymbolAddress(reinterpret_cast<void**>(&a.arrivals), HIP_SYMBOL(tcsl_arrivals))) != hipSuccess)
+                return static_cast<int>(e);
+            if (!a.arrivals)
+                return static_cast<int>(hipErrorInvalidSymbol);
+            table[dev] = a;
+            known[dev].store(true, std::memory_order_release);
+        }
+    }
+    *out = table[dev];
+    return 0;
+}
+
 template<int NB, bool HALF, bool BLDS, bool KSPLIT, bool ROWMAJ, int MAXW>
 int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const void* B, void* out, int M, int N,
                 int K, int split_k, int waves, unsigned lds_bytes, int ldb, int ldo, int relu, void* fused_out,
-                int ldc, int fuse_page, int dense_waves)
+                int ldc, unsigned int* arrivals, int dense_waves)
 {
     if (waves < 1 || waves > MAXW || lds_bytes > kMaxLdsBytes)
         return static_cast<int>(hipErrorInvalidValue);
@@ -935,7 +973,7 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
     hipLaunchKernelGGL(kernel, dim3(groups, split_k), dim3(waves * kWave), lds_bytes, stream,
                        offsets, static_cast<const u32x4*>(items), static_cast<const _Float16*>(B),
                        static_cast<_Float16*>(out), K, (nkb - 1) / split_k + 1, waves | dense_waves << 8, ldb, M, ldo,
-                       static_cast<_Float16*>(fused_out), ldc, fuse_page, relu, split_k);
+                       static_cast<_Float16*>(fused_out), arrivals, ldc, relu, split_k);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -953,7 +991,7 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
 // waves = 1..8 for N <= 32, 1..4 for N = 64; lds_bytes = what the shape needs (the host plans it).
 // ldb, ldo: token strides of B and of the output in elements (column-major; multiples of 8).
 // fuse_page >= 0: out = Split_K dense slabs, and the kernel itself reduces them into fused_out
-// (token stride ldc), counting arrivals on that page of counters; at most 4096 row groups.
+// (token stride ldc), counting arrivals on that page of counters (0 .. 255); at most 4096 row groups.
 // relu: bit 0 clamps final results at zero; with fuse_page >= 0, bits 8 and up = number of further
 // slabs behind the Split_K of this launch that the fused reduction adds as well.
 // dense_waves (mode 1; 0 = off): of the `waves` launched, only this many work on a unit whose
@@ -968,14 +1006,19 @@ extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offs
         return static_cast<int>(hipErrorInvalidValue);
     if (stage_b && (mode == 1 || row_major || N > 16))
         return static_cast<int>(hipErrorInvalidValue);
+    unsigned int* arrivals = nullptr;
     if (fuse_page >= 0) {
         const long groups = mode ? M / kTileRows : (M / kTileRows + waves - 1) / waves;
         if (fuse_page >= kCounterPages || groups > kCountersPerPage || row_major || split_k + (relu >> 8) < 2 || !fused_out)
             return static_cast<int>(hipErrorInvalidValue);
+        DeviceArrays a;
+        if (const int rc = device_arrays(&a))
+            return rc;
+        arrivals = a.arrivals + static_cast<size_t>(fuse_page) * kCountersPerPage;
     }
 #define TCSL_GO(NB, HALF, BLDS, KS, RM, MAXW) \
     launch_spmm<NB, HALF, BLDS, KS, RM, MAXW>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes, ldb, ldo, relu, \
-                                              fused_out, ldc, fuse_page, dense_waves)
+                                              fused_out, ldc, arrivals, dense_waves)
 #define TCSL_PICK(NB, HALF, MAXW)                                                                     \
     (row_major ? (mode ? TCSL_GO(NB, HALF, false, true, true, MAXW) : TCSL_GO(NB, HALF, false, false, true, MAXW)) \
                : (mode ? TCSL_GO(NB, HALF, false, true, false, MAXW) : TCSL_GO(NB, HALF, false, false, false, MAXW)))
@@ -1015,6 +1058,40 @@ extern "C" int tcsl_launch_copy(void* stream, void* dst, const void* src, long b
     hipLaunchKernelGGL(tcsl_copy_kernel, dim3(256 * 16), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), bytes / 16);
     return static_cast<int>(hipGetLastError());
+}
+
+// 1 and *id = the capture's id while `stream` is recording into a graph, 0 while it is not,
+// -1 when the runtime cannot say (treated by the caller like a capture it knows nothing about).
+extern "C" int tcsl_stream_capture(void* stream, unsigned long long* id)
+{
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    unsigned long long cid = 0;
+    if (hipStreamGetCaptureInfo(static_cast<hipStream_t>(stream), &st, &cid) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    if (st == hipStreamCaptureStatusNone)
+        return 0;
+    if (st != hipStreamCaptureStatusActive)
+        return -1;
+    *id = cid;
+    return 1;
+}
+
+// 1 when everything enqueued on `stream` has finished or the handle names no live stream any
+// more, 0 while work is pending (or the stream is capturing, or the runtime cannot say).
+extern "C" int tcsl_stream_idle(void* stream)
+{
+    // (a stream that is recording must not be queried: that would invalidate its capture)
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &st) == hipSuccess && st != hipStreamCaptureStatusNone)
+        return 0;
+    (void)hipGetLastError();
+    const hipError_t e = hipStreamQuery(static_cast<hipStream_t>(stream));
+    if (e == hipSuccess)
+        return 1;
+    (void)hipGetLastError();
+    return e == hipErrorContextIsDestroyed || e == hipErrorInvalidHandle ? 1 : 0;
 }
 
 // Timing events for benchmarks (the host logic never includes HIP headers).

@@ -318,7 +318,11 @@ int encode_file(const char* dense, int M, int K, const char* nz_path, const char
         out_sizes.write(reinterpret_cast<const char*>(&num_offsets), sizeof(int));
         out_nz.write(reinterpret_cast<const char*>(items), static_cast<std::streamsize>(sizeof(uint32_t)) * nnz);
         out_off.write(reinterpret_cast<const char*>(offs), static_cast<std::streamsize>(sizeof(int)) * num_offsets);
-        if (!out_sizes.good() || !out_nz.good() || !out_off.good())
+        // a short write may only show when the buffers are flushed: close first, then look
+        out_sizes.close();
+        out_nz.close();
+        out_off.close();
+        if (out_sizes.fail() || out_nz.fail() || out_off.fail())
             rc = kErrFile;
     }
     std::free(items);

@@ -62,6 +62,32 @@ def build_layer(G, torch, dev, h, N, sparsity, seed, keep_dense=False, weight_sc
     return Layer(mats), dense
 
 
+def build_layer_on_device(G, torch, dev, h, N, sparsity, seed, weight_std=0.02, sample_rows=0):
+    """One block with random-init weights made and encoded on the GPU (nothing crosses PCIe).
+
+    Every matrix is N(0, weight_std) fp16 with Bernoulli(1 - sparsity) kept entries, drawn from a
+    torch generator seeded with `seed`, and goes through the device encoder (same bits as the host
+    encoder would give for the same matrix).  With sample_rows > 0 the second value maps each
+    matrix name to (row indices, those rows of the dense matrix as a host fp16 array), for
+    checking products against a CPU reference without keeping the dense matrices.
+    """
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    mats, samples = {}, {}
+    for name, (M, K) in layer_shapes(h).items():
+        A = torch.randn((M, K), generator=gen, device=dev, dtype=torch.float32)
+        A.mul_(weight_std)
+        A.mul_(torch.rand((M, K), generator=gen, device=dev) >= sparsity)
+        A = A.to(torch.float16)
+        items, offsets = G.encode_on_device(A)
+        mats[name] = (items, offsets, M, K, G.SpMM_SuggestSplitK(M, N, K))
+        if sample_rows:
+            rows = torch.randperm(M, generator=gen, device=dev)[:sample_rows].sort().values
+            samples[name] = (rows.cpu().numpy(), A[rows].cpu().numpy())
+        del A, items
+    return Layer(mats), samples
+
+
 class Stack:
     def __init__(self, G, torch, layers, h, N):
         self.G, self.torch, self.layers, self.h, self.N = G, torch, layers, h, N
@@ -107,8 +133,10 @@ def main():
     ap.add_argument("--sparsity", type=float, default=0.8)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--distinct-weights", action="store_true",
-                    help="synthesise and encode every layer separately (default: one layer, copied in HBM)")
+    ap.add_argument("--weights", choices=("device", "host", "copied"), default="device",
+                    help="device: every layer's weights are drawn and encoded on the GPU (default); host: drawn and "
+                         "encoded on the host by the library's generator and encoder; copied: one host-made layer, "
+                         "copied in HBM for the others")
     ap.add_argument("--model-dir", help="run rank 0 of a converted one-rank model directory (<dir>/1-gpu/, written by "
                                         "graphneuralnetproj_amd.model_files) instead of synthetic weights")
     args = ap.parse_args()
@@ -130,11 +158,14 @@ def main():
         args.layers, h = model_files.read_config(rank_dir)
         layers = model_files.upload_layers(model_files.load_rank(rank_dir, 0, 1), dev, tokens=N)
     else:
-        first, _ = build_layer(G, torch, dev, h, N, args.sparsity, seed=1)
-        layers = [first]
-        for i in range(1, args.layers):
-            layers.append(build_layer(G, torch, dev, h, N, args.sparsity, seed=1 + i)[0] if args.distinct_weights
-                          else first.clone())
+        if args.weights == "device":
+            layers = [build_layer_on_device(G, torch, dev, h, N, args.sparsity, seed=1 + i)[0] for i in range(args.layers)]
+        else:
+            first, _ = build_layer(G, torch, dev, h, N, args.sparsity, seed=1)
+            layers = [first]
+            for i in range(1, args.layers):
+                layers.append(build_layer(G, torch, dev, h, N, args.sparsity, seed=1 + i)[0] if args.weights == "host"
+                              else first.clone())
     torch.cuda.synchronize()
     prep_s = time.perf_counter() - t0
     stack = Stack(G, torch, layers, h, N)
@@ -189,8 +220,10 @@ def main():
         "eager_ms": eager_ms, "graph_ms": graph_ms, "graph_matches_eager": graph_matches,
         "config": {"workload": f"{args.layers} layers x (QKV, out-proj, FFN1+ReLU, FFN2), h={h}, N={N}, "
                                f"{args.sparsity * 100:.0f}% sparse",
-                   "weights": "model directory" if args.model_dir else "distinct per layer" if args.distinct_weights
-                   else "one layer's weights copied per layer"},
+                   "weights": "model directory" if args.model_dir else
+                   {"device": "random-init per layer, drawn and encoded on the GPU",
+                    "host": "random-init per layer, drawn and encoded on the host",
+                    "copied": "one layer's weights copied per layer"}[args.weights]},
         "resident_weight_bytes": weight_bytes,
         "hbm_gbps": weight_bytes / (best_ms * 1e-3) / 1e9,
         "hbm_frac_of_peak": weight_bytes / (best_ms * 1e-3) / 1e9 / 8000.0,

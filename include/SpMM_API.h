@@ -86,10 +86,14 @@ SPMM_EXPORT int InitSparseMatrixA_API_NoReorder(const uint16_t* A_h, int M, int 
  * {8, 16, 32, 64} (csrc/SpMM_API.cu:192-193); hipErrorInvalidValue for M % 128,
  * K % 64, Split_K < 1, Split_K > 65535 or a null pointer (the reference checks these only in
  * debug builds, :93-98, and requires M % 256).  Nothing is launched on error.
- * Thread safe.  The in-launch reduction counts arrivals in a small static device array, one
- * page per stream handle (64 pages; further streams fall back to the second kernel): calls on
- * one stream never overlap, calls on different streams never share a page.  A call recorded
- * into a HIP graph keeps the page of the stream it was captured on.
+ * Thread safe.  The in-launch reduction counts arrivals in a static device array of counter
+ * pages (4 MiB per GPU), and two launches that might overlap never count on the same page:
+ * an eager call uses the page of its stream handle (64 pages; when all have owners, the least
+ * recently used one whose stream is idle or destroyed changes hands; if none is, this call runs
+ * the second kernel instead), a call recorded into a HIP graph the page of its (capture, stream)
+ * (192 pages, kept until the process ends, because the graph may be replayed at any time; beyond
+ * them captured calls run the second kernel).  What remains the caller's duty: two executable
+ * graphs instantiated from the same capture must not run at the same time.
  */
 SPMM_EXPORT int SpMM_SplitK_API(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets, const void* B,
                     void* C, int M_Global, int N_Global, int K_Global, void* Reduction_Workspace, int Split_K);

@@ -1,0 +1,33 @@
+// C handle on tcsl::CounterPages for tests/test_counter_pages.py (built by the test with g++).
+// "Streams" are arbitrary integers; the set of busy ones is what the test says it is.
+#include <set>
+
+#include "../../graphneuralnetproj_amd/csrc/counter_pages.h"
+
+namespace {
+std::set<void*> busy;
+bool idle(void* s) { return busy.count(s) == 0; }
+}  // namespace
+
+extern "C" {
+void* cp_new() { return new tcsl::CounterPages(); }
+void cp_delete(void* p) { delete static_cast<tcsl::CounterPages*>(p); }
+void cp_set_busy(unsigned long stream, int is_busy)
+{
+    if (is_busy)
+        busy.insert(reinterpret_cast<void*>(stream));
+    else
+        busy.erase(reinterpret_cast<void*>(stream));
+}
+int cp_acquire(void* p, unsigned long stream, int capturing, unsigned long long capture_id)
+{
+    tcsl::CounterPages* pages = static_cast<tcsl::CounterPages*>(p);
+    std::lock_guard<std::mutex> lock(pages->mutex());
+    return pages->acquire(reinterpret_cast<void*>(stream), capturing != 0, capture_id, idle);
+}
+int cp_eager_in_use(void* p) { return static_cast<tcsl::CounterPages*>(p)->eager_in_use(); }
+int cp_capture_in_use(void* p) { return static_cast<tcsl::CounterPages*>(p)->capture_in_use(); }
+int cp_eager_pages() { return tcsl::CounterPages::kEagerPages; }
+int cp_capture_pages() { return tcsl::CounterPages::kCapturePages; }
+int cp_eviction_tries() { return tcsl::CounterPages::kEvictionTries; }
+}

@@ -770,3 +770,121 @@ def test_short_segments_on_sparse_tile_rows(spmm, oracle, N, split_k, mode, wave
                                      waves, stage_b, 0, flags)
         torch.cuda.synchronize()
         assert_close(d_C.cpu().numpy(), ref)
+
+
+def _hip_runtime():
+    """The HIP runtime this process already holds (torch's), for making and destroying raw streams."""
+    import ctypes
+
+    _torch()
+    with open("/proc/self/maps") as f:
+        paths = {line.split()[-1] for line in f if "libamdhip64" in line}
+    assert len(paths) == 1, paths
+    hip = ctypes.CDLL(paths.pop())
+    hip.hipStreamCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+    hip.hipStreamDestroy.argtypes = [ctypes.c_void_p]
+    hip.hipStreamSynchronize.argtypes = [ctypes.c_void_p]
+    return hip
+
+
+def _fused_case(spmm, M=1024, K=2048, N=16, split_k=4, seed=321):
+    """Device operands of a call that takes the in-launch reduction (K-splitting launch, Split_K > 1),
+    and the bits of the same call with the reduction as a second kernel."""
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    A, B, items, offsets = make_case(spmm, M, K, N, 0.8, seed=seed)
+    d_items = torch.from_numpy(items.view(np.int32).copy()).to(dev)
+    d_offs = torch.from_numpy(offsets.copy()).to(dev)
+    d_B = torch.from_numpy(np.ascontiguousarray(B).view(np.int16).copy()).to(dev)
+    d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device=dev)
+    d_W = torch.full((split_k, N, M), float("nan"), dtype=torch.float16, device=dev)
+    spmm.SpMM_SplitK_API_Planned(None, d_items, d_offs, d_B, d_C, M, N, K, d_W, split_k, 1, 4, 0, 0,
+                                 spmm.SPMM_FLAG_SEPARATE_REDUCTION)
+    torch.cuda.synchronize()
+    return (d_items, d_offs, d_B, M, N, K, split_k), d_C.cpu().numpy().view(np.uint16)
+
+
+def test_fused_reduction_with_many_short_lived_streams(spmm):
+    """More stream handles than there are counter pages, each used once and destroyed: every call
+    must still give the bits of the separate reduction (pages of idle or destroyed streams change
+    hands; a call that finds none runs the second kernel)."""
+    import ctypes
+
+    torch = _torch()
+    hip = _hip_runtime()
+    (d_items, d_offs, d_B, M, N, K, split_k), want = _fused_case(spmm)
+    print("[gpu case] fused reduction on 200 short-lived streams", flush=True)
+    for i in range(200):
+        s = ctypes.c_void_p()
+        assert hip.hipStreamCreate(ctypes.byref(s)) == 0
+        d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device="cuda:0")
+        d_W = torch.full((split_k, N, M), float("nan"), dtype=torch.float16, device="cuda:0")
+        torch.cuda.synchronize()
+        spmm.SpMM_SplitK_API_Planned(s.value, d_items, d_offs, d_B, d_C, M, N, K, d_W, split_k, 1, 4, 0, 0, 0)
+        assert hip.hipStreamSynchronize(s) == 0
+        assert np.array_equal(d_C.cpu().numpy().view(np.uint16), want), f"stream {i}"
+        assert hip.hipStreamDestroy(s) == 0
+
+
+def test_fused_reduction_with_more_live_streams_than_pages(spmm):
+    """96 streams alive at once, calls dealt round robin without waiting: streams beyond the pages
+    get one only when an owner has gone idle, else the second kernel; same bits either way."""
+    import ctypes
+
+    torch = _torch()
+    hip = _hip_runtime()
+    (d_items, d_offs, d_B, M, N, K, split_k), want = _fused_case(spmm, seed=322)
+    streams, outs = [], []
+    for i in range(96):
+        s = ctypes.c_void_p()
+        assert hip.hipStreamCreate(ctypes.byref(s)) == 0
+        streams.append(s)
+        outs.append((torch.full((N, M), float("nan"), dtype=torch.float16, device="cuda:0"),
+                     torch.full((split_k, N, M), float("nan"), dtype=torch.float16, device="cuda:0")))
+    torch.cuda.synchronize()
+    print("[gpu case] fused reduction on 96 live streams", flush=True)
+    for rep in range(3):
+        for s, (d_C, d_W) in zip(streams, outs):
+            spmm.SpMM_SplitK_API_Planned(s.value, d_items, d_offs, d_B, d_C, M, N, K, d_W, split_k, 1, 4, 0, 0, 0)
+    for s in streams:
+        assert hip.hipStreamSynchronize(s) == 0
+    for i, (d_C, _) in enumerate(outs):
+        assert np.array_equal(d_C.cpu().numpy().view(np.uint16), want), f"stream {i}"
+    for s in streams:
+        assert hip.hipStreamDestroy(s) == 0
+
+
+def test_graph_replay_beside_eager_calls_on_the_capture_stream(spmm):
+    """A graph captured on stream S keeps counting on its own page: replays on another stream run
+    while eager calls with the in-launch reduction are queued on S, and both give the right bits."""
+    torch = _torch()
+    (d_items, d_offs, d_B, M, N, K, split_k), want = _fused_case(spmm, M=2048, K=4096, seed=323)
+    dev = torch.device("cuda:0")
+    mk = lambda: (torch.full((N, M), float("nan"), dtype=torch.float16, device=dev),
+                  torch.full((split_k, N, M), float("nan"), dtype=torch.float16, device=dev))
+    (gC, gW), (eC, eW) = mk(), mk()
+    S, other = torch.cuda.Stream(), torch.cuda.Stream()
+
+    def call(stream, C, W):
+        spmm.SpMM_SplitK_API_Planned(stream, d_items, d_offs, d_B, C, M, N, K, W, split_k, 1, 4, 0, 0, 0)
+
+    call(S, eC, eW)  # eager first: arms the kernel's attributes, gives S its eager page
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(S):
+        with torch.cuda.graph(g, stream=S):
+            for _ in range(4):
+                call(torch.cuda.current_stream(), gC, gW)
+    torch.cuda.synchronize()
+    print("[gpu case] graph replays on one stream beside eager calls on the capture stream", flush=True)
+    for rep in range(5):
+        gC.fill_(float("nan"))
+        eC.fill_(float("nan"))
+        torch.cuda.synchronize()
+        with torch.cuda.stream(other):
+            g.replay()
+        for _ in range(8):
+            call(S, eC, eW)
+        torch.cuda.synchronize()
+        assert np.array_equal(gC.cpu().numpy().view(np.uint16), want), f"replay {rep}"
+        assert np.array_equal(eC.cpu().numpy().view(np.uint16), want), f"eager beside replay {rep}"
