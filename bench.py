@@ -6,14 +6,24 @@ inputs already resident in HBM.  The compressed weight is held in several
 distinct HBM copies that the steps rotate through, so the stream cannot be
 served from the 256 MB Infinity Cache.
 
+The clocks are settled by the benchmark itself: before the --warmup steps it launches the
+same call, untimed, for at least PREWARM_SECONDS (reported as prewarm_launches), so a short
+--steps/--warmup run measures the same machine state as a long one.  The block of --steps
+steps, bracketed by synchronisations, is then timed --repeats times and the median reported.
+
 Prints ONE JSON line:
   value           effective TFLOPS, 2*M*N*K / step time (whole call)
   hbm_gbps        compressed-weight bytes / step time
   roofline        the main kernel alone: algorithmic bytes (16 * TileOffsets[last])
                   / its average duration, from two HIP events recorded on the launch
-                  stream around K back-to-back launches of it, against the 8 TB/s HBM peak
+                  stream around K back-to-back launches of it (median of --repeats such
+                  blocks), against the 8 TB/s HBM peak
   cpu_baseline    the CPU path timed on this host: reference encoder (oracle/_ref,
                   single thread) + fp32-accumulate dense GEMM (oracle, single thread)
+  sweep           the benchmark's other configurations, each timed for a fraction of a
+                  second after the headline (events around whole calls): ms per call and
+                  the fraction of 8 TB/s on that weight's compressed bytes; last, the
+                  64-layer decoder stack's time per token step
 
 One GPU only: --gpus above 1 exits with a message.
 """
@@ -37,6 +47,9 @@ MEASURED_TRAFFIC_BYTES = {
     ("opt30b_ffn1", 16, 1): 168.70e6,  # mode 1: no partial sums
     ("opt30b_ffn1", 16, 8): 175.50e6,  # mode 0: plus 7.34 MB of partial sums
 }
+TRAFFIC_SOURCE = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, scaled by a copy kernel of known "
+                  "size; summary in profiles/tcsl_spmm_kernel_opt30b_ffn1_n16_pmc.txt (not measured live)")
+PREWARM_SECONDS = 0.3
 FP16_MFMA_PEAK_TFLOPS = 2500.0
 
 WORKLOADS = {
@@ -86,7 +99,8 @@ def cpu_baseline(A, B, M, N, K, max_seconds=30.0):
     # the same GEMM spread over the host's cores by 128-row blocks (ctypes releases the GIL)
     from concurrent.futures import ThreadPoolExecutor
 
-    threads = max(1, min(16, os.cpu_count() or 1))
+    nproc = os.cpu_count() or 1
+    threads = max(1, min(16, nproc))
     blocks = [(r, min(r + 128, rows)) for r in range(0, rows, 128)]
     t0 = time.perf_counter()
     with ThreadPoolExecutor(threads) as pool:
@@ -97,6 +111,8 @@ def cpu_baseline(A, B, M, N, K, max_seconds=30.0):
         "unit": "TFLOPS",
         "cores": 1,
         "kind": "port",
+        "kinds": {"gemm": "port (oracle/tiled_csl_oracle.c)", "encode": f"{enc_kind}" + (" (oracle/_ref)" if enc_kind == "reference" else "")},
+        "nproc": nproc,
         "sample": (f"fp32-accumulate dense GEMM (oracle C loop) on the first {rows} of {M} rows, scaled to M; "
                    f"Tiled-CSL encode of the full matrix by the {enc_kind} encoder took {t_enc:.2f} s"),
         "gemm_s": t_gemm,
@@ -105,6 +121,147 @@ def cpu_baseline(A, B, M, N, K, max_seconds=30.0):
         "value_with_encode": flops / (t_gemm + t_enc) / 1e12,
         "all_cores": {"value": flops / t_gemm_mt / 1e12, "unit": "TFLOPS", "cores": threads, "gemm_s": t_gemm_mt},
     }
+
+
+def prewarm(call, torch, seconds=PREWARM_SECONDS):
+    """Launch call(i) back to back, untimed, until `seconds` of wall time have passed; returns the count."""
+    n = 0
+    t_end = time.perf_counter() + seconds
+    while time.perf_counter() < t_end:
+        for _ in range(100):
+            call(n)
+            n += 1
+        torch.cuda.synchronize()
+    return n
+
+
+def events_ms(lib, sptr, call, n):
+    """Milliseconds between two HIP events recorded on the launch stream around call(0) .. call(n-1)."""
+    ev0, ev1 = lib.SpMM_EventCreate(), lib.SpMM_EventCreate()
+    lib.SpMM_EventRecord(ev0, sptr)
+    for i in range(n):
+        call(i)
+    lib.SpMM_EventRecord(ev1, sptr)
+    ms = float(lib.SpMM_EventElapsedMs(ev0, ev1))
+    lib.SpMM_EventDestroy(ev0)
+    lib.SpMM_EventDestroy(ev1)
+    return ms
+
+
+SWEEP = [
+    # (label, workload, N, sparsity, row_skewed)
+    ("ffn1_n8", "opt30b_ffn1", 8, 0.8, False),
+    ("ffn1_n32", "opt30b_ffn1", 32, 0.8, False),
+    ("ffn1_n64", "opt30b_ffn1", 64, 0.8, False),
+    ("ffn1_70pct", "opt30b_ffn1", 16, 0.7, False),
+    ("ffn1_90pct", "opt30b_ffn1", 16, 0.9, False),
+    ("ffn1_skewed", "opt30b_ffn1", 16, 0.8, True),
+    ("ffn2", "opt30b_ffn2", 16, 0.8, False),
+    ("qkv", "opt30b_qkv", 16, 0.8, False),
+    ("outproj", "opt30b_outproj", 16, 0.8, False),
+    ("opt66b_qkv", "opt66b_qkv", 16, 0.8, False),
+    ("opt66b_outproj", "opt66b_outproj", 16, 0.8, False),
+    ("opt66b_ffn1", "opt66b_ffn1", 16, 0.8, False),
+    ("opt66b_ffn2", "opt66b_ffn2", 16, 0.8, False),
+]
+
+
+def sweep(G, lib, torch, dev, sptr, with_stack):
+    """The benchmark's other configurations: whole calls (main kernel + reduction) between two
+    events, 300 calls after a pre-warm, weights rotated over > 640 MB of copies."""
+    out = []
+    cache = {}
+    for label, workload, N, sparsity, skew in SWEEP:
+        M, K = WORKLOADS[workload][:2]
+        key = (workload, sparsity, skew)
+        if key not in cache:
+            cache.clear()  # one weight resident at a time
+            A = G.synth_weights(M, K, sparsity, skew, seed=1234)
+            items, offsets = G.InitSparseMatrixA_API(A)
+            del A
+            a_bytes = 16 * int(offsets[-1])
+            copies = min(64, max(2, -(-640 * 1024 * 1024 // max(a_bytes, 1))))
+            d_items = [torch.from_numpy(items.view(np.int32)).to(dev)]
+            d_items += [d_items[0].clone() for _ in range(copies - 1)]
+            d_offs = [torch.from_numpy(offsets).to(dev) for _ in range(copies)]
+            cache[key] = (a_bytes, copies, d_items, d_offs)
+        a_bytes, copies, d_items, d_offs = cache[key]
+        split_k = G.SpMM_SuggestSplitK(M, N, K)
+        d_B = torch.from_numpy(G.synth_activations(N, K, seed=4321).view(np.int16)).to(dev)
+        d_C = torch.zeros((N, M), dtype=torch.float16, device=dev)
+        d_W = torch.zeros((max(split_k, 1), N, M), dtype=torch.float16, device=dev)
+        p_items = [ctypes.c_void_p(t.data_ptr()) for t in d_items]
+        p_offs = [ctypes.c_void_p(t.data_ptr()) for t in d_offs]
+        p_B, p_C, p_W = (ctypes.c_void_p(t.data_ptr()) for t in (d_B, d_C, d_W))
+
+        def call(i):
+            rc = lib.SpMM_SplitK_API(sptr, None, p_items[i % copies], p_offs[i % copies], p_B, p_C, M, N, K, p_W, split_k)
+            if rc:
+                raise RuntimeError(f"SpMM_SplitK_API -> {rc}")
+
+        prewarm(call, torch, 0.1)
+        ms = float(np.median([events_ms(lib, sptr, call, 100) for _ in range(3)])) / 100
+        torch.cuda.synchronize()
+        plan = G.SpMM_PlanLaunch(M, N, K, split_k)
+        out.append({"case": label, "M": M, "K": K, "N": N, "sparsity": sparsity, "row_skewed": skew, "split_k": split_k,
+                    "plan": f"mode {plan['mode']}, {plan['waves']} waves", "compressed_bytes": a_bytes,
+                    "ms": ms, "frac": a_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                    "tflops": 2.0 * M * N * K / (ms * 1e-3) / 1e12})
+    cache.clear()
+    if with_stack:
+        out.append(stack_step(G, torch, dev))
+    return out
+
+
+def stack_step(G, torch, dev, layers=64, h=9216, N=16, sparsity=0.8):
+    """64 OPT-66B-shaped blocks, random-init weights drawn and encoded on the GPU (about 52 GB
+    resident): time per token step, eager and as a HIP graph."""
+    from graphneuralnetproj_amd import decoder_stack as DS
+
+    torch.cuda.empty_cache()
+    t0 = time.perf_counter()
+    blocks = [DS.build_layer_on_device(G, torch, dev, h, N, sparsity, seed=1 + i)[0] for i in range(layers)]
+    torch.cuda.synchronize()
+    build_s = time.perf_counter() - t0
+    stack = DS.Stack(G, torch, blocks, h, N)
+    x0 = torch.from_numpy(G.synth_activations(N, h, seed=99).view(np.int16)).to(dev).view(torch.float16)
+    stream = torch.cuda.current_stream()
+    stack.x[0].copy_(x0)
+    for _ in range(5):
+        stack.step(stream)
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        for _ in range(5):
+            stack.step(stream)
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) * 1e3 / 5)
+    eager_ms = float(np.median(times))
+    graph_ms = None
+    try:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            stack.step(torch.cuda.current_stream())
+        g.replay()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            for _ in range(5):
+                g.replay()
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) * 1e3 / 5)
+        graph_ms = float(np.median(times))
+    except Exception as e:  # the eager figure stands on its own
+        graph_ms = None
+        print(f"bench.py: graph capture of the stack failed: {e}", file=sys.stderr)
+    weight_bytes = sum(L.bytes() for L in blocks)
+    ms = min(eager_ms, graph_ms) if graph_ms else eager_ms
+    return {"case": "decoder_stack", "layers": layers, "hidden": h, "N": N, "sparsity": sparsity,
+            "weights": "random-init per layer, drawn and encoded on the GPU", "resident_weight_bytes": weight_bytes,
+            "ms": ms, "eager_ms": eager_ms, "graph_ms": graph_ms, "frac": weight_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "hbm_floor_ms": weight_bytes / (HBM_PEAK_GBPS * 1e9) * 1e3, "build_s": build_s}
 
 
 def main():
@@ -121,6 +278,9 @@ def main():
     ap.add_argument("--copies", type=int, default=0, help="distinct HBM copies of the weight (0 = enough for > 640 MB)")
     ap.add_argument("--no-reorder", action="store_true",
                     help="encode with InitSparseMatrixA_API_NoReorder (the reference's ablation of its bank-aware reordering)")
+    ap.add_argument("--repeats", type=int, default=15, help="timed blocks of --steps steps; the median is reported")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the other configurations after the headline")
+    ap.add_argument("--no-stack", action="store_true", help="sweep without the 64-layer decoder stack (52 GB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
     ap.add_argument("--calibration-copies", type=int, default=0,
@@ -204,32 +364,36 @@ def main():
             print(json.dumps({"error": "parity check failed", "check": check}))
             sys.exit(1)
 
-    # ---- timed region: W warm-up steps, then exactly K steps between synchronisations
+    # ---- settle the clocks: the same call, untimed, for a fixed wall time whatever --warmup says
+    prewarm_launches = prewarm(step, torch)
+
+    # ---- timed region: W warm-up steps, then exactly K steps between synchronisations; that
+    # block is timed --repeats times (each with its own synchronisations) and the median reported
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(i)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
+    blocks_ms = []
+    for r in range(max(1, args.repeats)):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step(i)
+        torch.cuda.synchronize()
+        blocks_ms.append((time.perf_counter() - t0) * 1e3)
+    ms_per_step = float(np.median(blocks_ms)) / args.steps
 
     # ---- the main kernel alone, live: K back-to-back launches of it (no reduction in between)
     # bracketed by two HIP events recorded on the launch stream; the average includes the
     # dispatch gap between consecutive kernels but no per-launch event overhead.
-    for i in range(min(args.warmup, 200)):
-        lib.SpMM_SplitK_Partials(sptr, p_items[i % copies], p_offs[i % copies], p_B, p_W, M, N, K, split_k)
-    ev0, ev1 = lib.SpMM_EventCreate(), lib.SpMM_EventCreate()
-    lib.SpMM_EventRecord(ev0, sptr)
-    for i in range(args.steps):
+    def partials(i):
         rc = lib.SpMM_SplitK_Partials(sptr, p_items[i % copies], p_offs[i % copies], p_B, p_W, M, N, K, split_k)
         if rc:
             raise RuntimeError(f"SpMM_SplitK_Partials -> {rc}")
-    lib.SpMM_EventRecord(ev1, sptr)
-    kernel_ms_avg = float(lib.SpMM_EventElapsedMs(ev0, ev1)) / args.steps
-    lib.SpMM_EventDestroy(ev0)
-    lib.SpMM_EventDestroy(ev1)
+
+    for i in range(200):
+        partials(i)
+    kernel_blocks_ms = [events_ms(lib, sptr, partials, args.steps) for _ in range(max(1, args.repeats))]
+    kernel_ms_avg = float(np.median(kernel_blocks_ms)) / args.steps
     torch.cuda.synchronize()
 
     for i in range(args.calibration_copies):
@@ -242,14 +406,20 @@ def main():
     flops = 2.0 * M * N * K
     tflops = flops / (ms_per_step * 1e-3) / 1e12
     kernel_gbps = a_bytes / (kernel_ms_avg * 1e-3) / 1e9
+    default_workload = (args.workload == "opt30b_ffn1" and N == 16 and sparsity == 0.8 and not skew)
     out = {
-        "metric": "SpMM eff. TFLOPS + HBM GB/s (% roofline), OPT-30B FFN1 80% sparse, N=16",
+        "metric": ("SpMM eff. TFLOPS + HBM GB/s (% roofline), OPT-30B FFN1 80% sparse, N=16" if default_workload else
+                   f"SpMM eff. TFLOPS + HBM GB/s (% roofline), {args.workload} {sparsity * 100:.0f}% sparse"
+                   f"{' (row-skewed)' if skew else ''}, N={N}"),
         "value": tflops,
         "unit": "TFLOPS",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_per_step,
+        "timing": {"repeats": len(blocks_ms), "statistic": "median of the timed blocks of --steps steps",
+                   "block_ms_min": float(min(blocks_ms)), "block_ms_max": float(max(blocks_ms)),
+                   "prewarm_launches": prewarm_launches, "prewarm_seconds": PREWARM_SECONDS},
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -277,6 +447,7 @@ def main():
             "frac": kernel_gbps / HBM_PEAK_GBPS,
             "traffic": (MEASURED_TRAFFIC_BYTES.get((args.workload, N, split_k))
                         if sparsity == 0.8 and not skew else None),
+            "traffic_source": TRAFFIC_SOURCE,
             "kernel": "tcsl_spmm_kernel",
             "kernel_ms_avg": kernel_ms_avg,
             "algorithmic_bytes_per_launch": a_bytes,
@@ -286,6 +457,10 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(A, B, M, N, K)
+    if not args.no_sweep:
+        del d_items, d_offs, p_items, p_offs
+        torch.cuda.empty_cache()
+        out["sweep"] = sweep(G, lib, torch, dev, sptr, with_stack=not args.no_stack)
     print(json.dumps(out))
 
 

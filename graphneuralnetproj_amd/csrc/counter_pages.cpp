@@ -23,17 +23,17 @@ int CounterPages::acquire(void* stream, bool capturing, unsigned long long captu
         eager_[eager_used_] = Eager{stream, clock_};
         return eager_used_++;
     }
-    // All pages have an owner: look at the least recently used ones, oldest first, and take the
-    // first whose stream has nothing left to run.
+    // All pages have an owner: look at the least recently used recycled ones, oldest first, and
+    // take the first whose last launch has finished.
     uint64_t newer_than = 0;
     for (int t = 0; t < kEvictionTries; t++) {
         int oldest = -1;
-        for (int i = 0; i < kEagerPages; i++)
+        for (int i = kPermanentPages; i < kEagerPages; i++)
             if (eager_[i].last_use > newer_than && (oldest < 0 || eager_[i].last_use < eager_[oldest].last_use))
                 oldest = i;
         if (oldest < 0)
             break;
-        if (idle && idle(eager_[oldest].stream)) {
+        if (idle && idle(oldest)) {
             eager_[oldest] = Eager{stream, clock_};
             return oldest;
         }

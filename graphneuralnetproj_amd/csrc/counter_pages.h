@@ -1,6 +1,6 @@
 // Who counts where: hands out the pages of arrival counters that the in-launch split-K
-// reduction of the main kernel needs.  Host only, no GPU calls of its own (the two questions it
-// has about a stream are asked through function pointers, so the logic runs in a CPU test).
+// reduction of the main kernel needs.  Host only, no GPU calls of its own (the one question it
+// has about the GPU is asked through a function pointer, so the logic runs in a CPU test).
 //
 // A page is a row of device counters, all zero between launches (the last workgroup to arrive
 // sets its counter back).  Two launches may share a page only if they cannot overlap in time:
@@ -8,8 +8,11 @@
 //   * calls captured into one graph on one stream are   -> one page per (capture, stream),
 //     ordered in every replay of that graph                held for as long as the process runs,
 //                                                          because the graph may be replayed at any time.
-// Eager pages are recycled: when none is free, the least recently used page whose stream is
-// idle (or no longer exists) changes hands.  A stream that is still busy keeps its page.
+// The first kPermanentPages stream handles keep their page for good.  Later handles share
+// kRecycledPages pages that change hands: when none is free, the least recently used one whose
+// last launch has finished goes to the newcomer.  Whether it has finished is asked of an event
+// that the caller records behind every launch on such a page; a stream handle is never handed
+// back to the runtime by this class or on its behalf (the stream may long have been destroyed).
 // When nothing can be had the caller runs the reduction as a kernel of its own.
 #pragma once
 
@@ -20,19 +23,24 @@ namespace tcsl {
 
 class CounterPages {
 public:
-    static constexpr int kEagerPages = 64;
+    static constexpr int kPermanentPages = 32;
+    static constexpr int kRecycledPages = 32;
+    static constexpr int kEagerPages = kPermanentPages + kRecycledPages;
     static constexpr int kCapturePages = 192;
     static constexpr int kPages = kEagerPages + kCapturePages;
     static constexpr int kEvictionTries = 8;  // least recently used pages looked at when none is free
 
-    // true: everything enqueued on the stream has finished, or the handle names no stream any more
-    using IdleFn = bool (*)(void* stream);
+    // true: the last launch that counted on this (recycled) page has finished
+    using IdleFn = bool (*)(int page);
 
     // Page (0 .. kPages-1) for a call about to be enqueued on `stream`, or -1.  capturing: the
     // stream is recording into a graph, capture_id names the capture.  The caller holds mutex()
-    // from before this call until its launch has been enqueued, so that a page cannot change
-    // hands between being looked up and being used.
+    // from before this call until its launch has been enqueued and, if recycled(page), the
+    // page's event recorded behind it, so that a page cannot change hands in between.
     int acquire(void* stream, bool capturing, unsigned long long capture_id, IdleFn idle);
+
+    // Pages whose every launch must be followed by the event that `idle` looks at.
+    static constexpr bool recycled(int page) { return page >= kPermanentPages && page < kEagerPages; }
 
     std::mutex& mutex() { return mu_; }
 

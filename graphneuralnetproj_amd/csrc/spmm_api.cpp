@@ -27,7 +27,9 @@ int a24_launch_split_pack(void* stream, const void* A, void* packed, void* resid
 int a24_side_begin(void* stream, void** side);
 int a24_side_end(void* stream, void* side);
 int tcsl_stream_capture(void* stream, unsigned long long* id);
-int tcsl_stream_idle(void* stream);
+int tcsl_page_prepare(int page);
+int tcsl_page_mark(int page, void* stream);
+int tcsl_page_idle(int page);
 void* tcsl_event_create(void);
 void tcsl_event_destroy(void* e);
 int tcsl_event_record(void* e, void* stream);
@@ -121,7 +123,11 @@ int counter_page(void* stream)
     const int capturing = tcsl_stream_capture(stream, &capture_id);
     if (capturing < 0)
         return -1;
-    return counter_pages().acquire(stream, capturing == 1, capture_id, [](void* s) { return tcsl_stream_idle(s) == 1; });
+    const int page = counter_pages().acquire(stream, capturing == 1, capture_id, [](int p) { return tcsl_page_idle(p) == 1; });
+    // a page that changes hands is guarded by an event behind each of its launches; without one, no page
+    if (page >= 0 && tcsl::CounterPages::recycled(page) && tcsl_page_prepare(page) != 0)
+        return -1;
+    return page;
 }
 
 // What varies between the entry points that end in the same two launches.
@@ -169,11 +175,14 @@ int launch_main(void* stream, const void* Compressed_A, const int* TileOffsets, 
             dense_waves = p.waves;
         }
     }
-    return tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, out, M, N, K, Split_K, run.mode, run.waves, run.stage_b,
-                            o.row_major ? 1 : 0, run.lds_bytes, ldb, ldo,
-                            (relu && (Split_K == 1 || page >= 0) ? 1 : 0)  // slabs of partial sums are never clamped
-                                | (page >= 0 ? o.extra_slabs << 8 : 0),
-                            page >= 0 ? fused_out : nullptr, static_cast<int>(ldc), page, dense_waves);
+    int rc = tcsl_launch_spmm(stream, Compressed_A, TileOffsets, B, out, M, N, K, Split_K, run.mode, run.waves, run.stage_b,
+                              o.row_major ? 1 : 0, run.lds_bytes, ldb, ldo,
+                              (relu && (Split_K == 1 || page >= 0) ? 1 : 0)  // slabs of partial sums are never clamped
+                                  | (page >= 0 ? o.extra_slabs << 8 : 0),
+                              page >= 0 ? fused_out : nullptr, static_cast<int>(ldc), page, dense_waves);
+    if (rc == 0 && tcsl::CounterPages::recycled(page))
+        rc = tcsl_page_mark(page, stream);
+    return rc;
 }
 
 int check_call(const void* Compressed_A, const int* TileOffsets, const void* B, const void* C, int M, int N, int K,

@@ -1078,20 +1078,64 @@ extern "C" int tcsl_stream_capture(void* stream, unsigned long long* id)
     return 1;
 }
 
-// 1 when everything enqueued on `stream` has finished or the handle names no live stream any
-// more, 0 while work is pending (or the stream is capturing, or the runtime cannot say).
-extern "C" int tcsl_stream_idle(void* stream)
+// Events behind the launches that count on a recycled counter page (the host's page table says
+// which pages those are): one event per page, made on first use, asked when the page is wanted
+// for another stream.  Only ever called with the page table's lock held.
+namespace {
+constexpr int kGuardedPages = 64;
+struct PageGuard {
+    hipEvent_t event;
+    int device;
+};
+PageGuard page_guards[kGuardedPages] = {};
+}  // namespace
+
+// Makes sure `page` has an event on the current device; 0 or a hipError_t value.
+extern "C" int tcsl_page_prepare(int page)
 {
-    // (a stream that is recording must not be queried: that would invalidate its capture)
-    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &st) == hipSuccess && st != hipStreamCaptureStatusNone)
+    if (page < 0 || page >= kGuardedPages)
+        return static_cast<int>(hipErrorInvalidValue);
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess)
+        return static_cast<int>(e);
+    PageGuard& g = page_guards[page];
+    if (g.event && g.device == dev)
         return 0;
-    (void)hipGetLastError();
-    const hipError_t e = hipStreamQuery(static_cast<hipStream_t>(stream));
+    if (g.event) {  // the page moved to a stream of another device (its last launch there has finished)
+        (void)hipEventDestroy(g.event);
+        g.event = nullptr;
+    }
+    if ((e = hipEventCreateWithFlags(&g.event, hipEventDisableTiming)) != hipSuccess) {
+        g.event = nullptr;
+        (void)hipGetLastError();
+        return static_cast<int>(e);
+    }
+    g.device = dev;
+    return 0;
+}
+
+// Records the page's event behind what `stream` holds so far.
+extern "C" int tcsl_page_mark(int page, void* stream)
+{
+    if (page < 0 || page >= kGuardedPages || !page_guards[page].event)
+        return static_cast<int>(hipErrorInvalidValue);
+    return static_cast<int>(hipEventRecord(page_guards[page].event, static_cast<hipStream_t>(stream)));
+}
+
+// 1 when the last launch marked on the page has finished (or none ever was), 0 while it has not
+// or the runtime cannot say.
+extern "C" int tcsl_page_idle(int page)
+{
+    if (page < 0 || page >= kGuardedPages)
+        return 0;
+    if (!page_guards[page].event)
+        return 1;
+    const hipError_t e = hipEventQuery(page_guards[page].event);
     if (e == hipSuccess)
         return 1;
     (void)hipGetLastError();
-    return e == hipErrorContextIsDestroyed || e == hipErrorInvalidHandle ? 1 : 0;
+    return 0;
 }
 
 // Timing events for benchmarks (the host logic never includes HIP headers).

@@ -88,12 +88,14 @@ SPMM_EXPORT int InitSparseMatrixA_API_NoReorder(const uint16_t* A_h, int M, int 
  * debug builds, :93-98, and requires M % 256).  Nothing is launched on error.
  * Thread safe.  The in-launch reduction counts arrivals in a static device array of counter
  * pages (4 MiB per GPU), and two launches that might overlap never count on the same page:
- * an eager call uses the page of its stream handle (64 pages; when all have owners, the least
- * recently used one whose stream is idle or destroyed changes hands; if none is, this call runs
- * the second kernel instead), a call recorded into a HIP graph the page of its (capture, stream)
- * (192 pages, kept until the process ends, because the graph may be replayed at any time; beyond
- * them captured calls run the second kernel).  What remains the caller's duty: two executable
- * graphs instantiated from the same capture must not run at the same time.
+ * an eager call uses the page of its stream handle (the first 32 handles keep theirs for good;
+ * later ones share 32 pages, each guarded by an event that the call records behind its launch,
+ * and when all have owners the least recently used one whose last launch has finished changes
+ * hands; if none has, this call runs the second kernel instead), a call recorded into a HIP graph
+ * the page of its (capture, stream) (192 pages, kept until the process ends, because the graph
+ * may be replayed at any time; beyond them captured calls run the second kernel).  What remains
+ * the caller's duty: two executable graphs instantiated from the same capture must not run at
+ * the same time.
  */
 SPMM_EXPORT int SpMM_SplitK_API(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets, const void* B,
                     void* C, int M_Global, int N_Global, int K_Global, void* Reduction_Workspace, int Split_K);

@@ -24,6 +24,7 @@ def cp(tmp_path_factory):
     lib.cp_acquire.argtypes = [ctypes.c_void_p, ctypes.c_ulong, ctypes.c_int, ctypes.c_ulonglong]
     lib.cp_eager_in_use.argtypes = [ctypes.c_void_p]
     lib.cp_capture_in_use.argtypes = [ctypes.c_void_p]
+    lib.cp_recycled.argtypes = [ctypes.c_int]
     return lib
 
 
@@ -59,47 +60,54 @@ def test_exhaustion_with_busy_streams_gives_no_page(cp, pages):
             cp.cp_set_busy(stream(i), 0)
 
 
-def test_idle_least_recently_used_page_changes_hands(cp, pages):
-    E = cp.cp_eager_pages()
+def test_first_streams_keep_their_pages_for_good(cp, pages):
+    """The pages of the first streams never change hands (no event is recorded behind their
+    launches, so nobody could tell when they are idle); only the later, recycled pages do."""
+    E, P = cp.cp_eager_pages(), cp.cp_permanent_pages()
     first = [cp.cp_acquire(pages, stream(i), 0, 0) for i in range(E)]
-    cp.cp_acquire(pages, stream(0), 0, 0)                     # stream 0 is now the most recent user
-    cp.cp_set_busy(stream(1), 1)                              # the oldest owner is busy ...
+    assert [cp.cp_recycled(p) for p in first] == [0] * P + [1] * (E - P)
+    for i in range(20 * E):                                   # a crowd of newcomers, everybody idle
+        assert cp.cp_recycled(cp.cp_acquire(pages, stream(1000 + i), 0, 0)) == 1
+    assert [cp.cp_acquire(pages, stream(i), 0, 0) for i in range(P)] == first[:P]
+
+
+def test_idle_least_recently_used_page_changes_hands(cp, pages):
+    E, P = cp.cp_eager_pages(), cp.cp_permanent_pages()
+    first = [cp.cp_acquire(pages, stream(i), 0, 0) for i in range(E)]
+    cp.cp_acquire(pages, stream(P), 0, 0)                     # the first recycled page's owner is now the most recent user
+    cp.cp_set_busy(stream(P + 1), 1)                          # the oldest remaining one is busy ...
     try:
         p = cp.cp_acquire(pages, stream(E), 0, 0)
-        assert p == first[2]                                  # ... so the next oldest idle one gives way
+        assert p == first[P + 2]                              # ... so the next oldest idle one gives way
         # the evicted stream comes back: it must not get the page its successor now counts on
         cp.cp_set_busy(stream(E), 1)
-        q = cp.cp_acquire(pages, stream(2), 0, 0)
+        q = cp.cp_acquire(pages, stream(P + 2), 0, 0)
         assert q != p and q >= 0
     finally:
-        cp.cp_set_busy(stream(1), 0)
+        cp.cp_set_busy(stream(P + 1), 0)
         cp.cp_set_busy(stream(E), 0)
 
 
 def test_many_short_lived_streams_always_get_a_page(cp, pages):
-    """A process that keeps making and destroying streams (every handle idle or gone when the next
-    appears) never falls off the fused path."""
+    """A process that keeps making and destroying streams (every launch finished when the next
+    stream appears) never falls off the fused path."""
     E = cp.cp_eager_pages()
-    owners = {}
     for i in range(10 * E):
-        p = cp.cp_acquire(pages, stream(i), 0, 0)
-        assert 0 <= p < E
-        owners[p] = i
-    assert len(owners) == E
+        assert 0 <= cp.cp_acquire(pages, stream(i), 0, 0) < E
 
 
 def test_eviction_looks_at_a_bounded_number_of_pages(cp, pages):
-    E, T = cp.cp_eager_pages(), cp.cp_eviction_tries()
+    E, P, T = cp.cp_eager_pages(), cp.cp_permanent_pages(), cp.cp_eviction_tries()
     for i in range(E):
         cp.cp_acquire(pages, stream(i), 0, 0)
-    for i in range(T):                                        # the T oldest are busy, the rest idle
+    for i in range(P, P + T):                                 # the T oldest recycled pages are busy, the rest idle
         cp.cp_set_busy(stream(i), 1)
     try:
         assert cp.cp_acquire(pages, stream(E), 0, 0) == -1
-        cp.cp_set_busy(stream(T - 1), 0)
+        cp.cp_set_busy(stream(P + T - 1), 0)
         assert cp.cp_acquire(pages, stream(E), 0, 0) >= 0
     finally:
-        for i in range(T):
+        for i in range(P, P + T):
             cp.cp_set_busy(stream(i), 0)
 
 
