@@ -26,6 +26,7 @@ int a24_launch_spmm(void* stream, const void* packed, const void* B, void* out, 
 int a24_launch_split_pack(void* stream, const void* A, void* packed, void* residual, int M, int K);
 int a24_side_begin(void* stream, void** side);
 int a24_side_end(void* stream, void* side);
+int tcsl_static_workspace(void** slabs, long* bytes);
 int tcsl_stream_capture(void* stream, unsigned long long* id);
 int tcsl_page_prepare(int page);
 int tcsl_page_mark(int page, void* stream);
@@ -130,6 +131,8 @@ int counter_page(void* stream)
     return page;
 }
 
+constexpr int kStaticWorkspacePage = 1 << 20;  // the counters inside the static workspace (spmm_kernels.hip: kScratchPage)
+
 // What varies between the entry points that end in the same two launches.
 struct CallOptions {
     bool row_major = false;   // B is [K][N], C and the slabs [M][N]
@@ -142,6 +145,7 @@ struct CallOptions {
     const tcsl::LaunchPlan* forced = nullptr;
     bool adaptive_waves = false;  // with `forced`: launch it the way a planned call would be
     int extra_slabs = 0;      // fused reduction only: slabs of an earlier launch, right behind this one's, to add as well
+    bool static_workspace = false;  // the slabs are the library's static workspace: count arrivals there too
 };
 
 // fused_out != nullptr asks for the fused reduction; *fused says whether it was possible.
@@ -158,8 +162,12 @@ int launch_main(void* stream, const void* Compressed_A, const int* TileOffsets, 
     // on its stream counts as busy and the page cannot change hands.
     std::unique_lock<std::mutex> page_lock;
     if (fused_out && p.mode == 1 && M / tcsl::kTileRows <= 4096) {
-        page_lock = std::unique_lock<std::mutex>(counter_pages().mutex());
-        page = counter_page(stream);
+        if (o.static_workspace) {
+            page = kStaticWorkspacePage;
+        } else {
+            page_lock = std::unique_lock<std::mutex>(counter_pages().mutex());
+            page = counter_page(stream);
+        }
     }
     if (fused)
         *fused = page >= 0;
@@ -196,6 +204,32 @@ extern "C" int SpMM_SplitK_API(void* stream, const void* A, const void* Compress
 {
     (void)A;
     return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, CallOptions{});
+}
+
+extern "C" int SpMM_SplitK_API_StaticWorkspace(void* stream, const void* A, const void* Compressed_A,
+                                               const int* TileOffsets, const void* B, void* C, int M, int N, int K,
+                                               int Split_K)
+{
+    (void)A;
+    void* slabs = nullptr;
+    long room = 0;
+    if (const int rc = check_call(Compressed_A, TileOffsets, B, C, M, N, K, true, Split_K))
+        return rc;
+    if (Split_K > 1) {
+        if (const int rc = tcsl_static_workspace(&slabs, &room))
+            return rc;
+        const long need = static_cast<long>(Split_K) * M * N * 2;
+        if (need > room) {
+            std::fprintf(stderr,
+                         "SpMM_SplitK_API_StaticWorkspace: Split_K=%d x M=%d x N=%d fp16 partial sums need %ld bytes, the "
+                         "static workspace holds %ld; use a smaller Split_K or SpMM_SplitK_API with a workspace of your own\n",
+                         Split_K, M, N, need, room);
+            return tcsl_error_invalid_value();
+        }
+    }
+    CallOptions o;
+    o.static_workspace = true;
+    return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, slabs, Split_K, o);
 }
 
 extern "C" int SpMM_SplitK_API_RowMajor(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets,

@@ -103,6 +103,15 @@ constexpr int kCounterPages = 256;
 constexpr int kCountersPerPage = 4096;
 static __device__ __align__(256) unsigned int tcsl_arrivals[kCounterPages][kCountersPerPage];
 
+// Workspace of the entry point that allocates nothing (SpMM_SplitK_API_StaticWorkspace): one
+// page of arrival counters, then room for the slabs of partial sums.  Every device the library
+// runs on holds its own copy for as long as the process lives.  In host code the name is only a
+// handle for hipGetSymbolAddress; kernels and launchers use the per-device address that call returns.
+constexpr int kScratchPage = 1 << 20;  // "page number" of the scratch's own counters
+constexpr size_t kScratchCounterBytes = kCountersPerPage * sizeof(unsigned int);
+constexpr size_t kScratchSlabBytes = size_t(32) << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchCounterBytes + kScratchSlabBytes];
+
 template<int... Is, typename F>
 __device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F&& f)
 {
@@ -910,11 +919,12 @@ __global__ __launch_bounds__(256) void tcsl_copy_kernel(u32x4* __restrict__ dst,
         dst[i] = src[i];
 }
 
-// Device address of the counter pages on the current device.  A __device__ array's name in
-// host code is a handle, not an address, and every device holds its own copy: the address is
-// asked for once per device (with that device current) and kept.
+// Device addresses of the two static arrays above on the current device.  A __device__ array's
+// name in host code is a handle, not an address, and every device holds its own copy: the
+// address is asked for once per device (with that device current) and kept.
 struct DeviceArrays {
     unsigned int* arrivals;      // tcsl_arrivals
+    unsigned char* scratch;      // scratch
 };
 constexpr int kMaxDevices = 64;
 int device_arrays(DeviceArrays* out)
@@ -931,10 +941,12 @@ int device_arrays(DeviceArrays* out)
     if (!known[dev].load(std::memory_order_acquire)) {
         std::lock_guard<std::mutex> lock(mu);
         if (!known[dev].load(std::memory_order_relaxed)) {
-            DeviceArrays a{nullptr};
+            DeviceArrays a{nullptr, nullptr};
             if ((e = hipGetSymbolAddress(reinterpret_cast<void**>(&a.arrivals), HIP_SYMBOL(tcsl_arrivals))) != hipSuccess)
                 return static_cast<int>(e);
-            if (!a.arrivals)
+            if ((e = hipGetSymbolAddress(reinterpret_cast<void**>(&a.scratch), HIP_SYMBOL(scratch))) != hipSuccess)
+                return static_cast<int>(e);
+            if (!a.arrivals || !a.scratch)
                 return static_cast<int>(hipErrorInvalidSymbol);
             table[dev] = a;
             known[dev].store(true, std::memory_order_release);
@@ -991,7 +1003,8 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
 // waves = 1..8 for N <= 32, 1..4 for N = 64; lds_bytes = what the shape needs (the host plans it).
 // ldb, ldo: token strides of B and of the output in elements (column-major; multiples of 8).
 // fuse_page >= 0: out = Split_K dense slabs, and the kernel itself reduces them into fused_out
-// (token stride ldc), counting arrivals on that page of counters (0 .. 255); at most 4096 row groups.
+// (token stride ldc), counting arrivals on that page of counters (0 .. 255: the library's pages;
+// kScratchPage: the counters of the static workspace); at most 4096 row groups.
 // relu: bit 0 clamps final results at zero; with fuse_page >= 0, bits 8 and up = number of further
 // slabs behind the Split_K of this launch that the fused reduction adds as well.
 // dense_waves (mode 1; 0 = off): of the `waves` launched, only this many work on a unit whose
@@ -1009,12 +1022,14 @@ extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offs
     unsigned int* arrivals = nullptr;
     if (fuse_page >= 0) {
         const long groups = mode ? M / kTileRows : (M / kTileRows + waves - 1) / waves;
-        if (fuse_page >= kCounterPages || groups > kCountersPerPage || row_major || split_k + (relu >> 8) < 2 || !fused_out)
+        if ((fuse_page >= kCounterPages && fuse_page != kScratchPage) || groups > kCountersPerPage || row_major ||
+            split_k + (relu >> 8) < 2 || !fused_out)
             return static_cast<int>(hipErrorInvalidValue);
         DeviceArrays a;
         if (const int rc = device_arrays(&a))
             return rc;
-        arrivals = a.arrivals + static_cast<size_t>(fuse_page) * kCountersPerPage;
+        arrivals = fuse_page == kScratchPage ? reinterpret_cast<unsigned int*>(a.scratch)
+                                             : a.arrivals + static_cast<size_t>(fuse_page) * kCountersPerPage;
     }
 #define TCSL_GO(NB, HALF, BLDS, KS, RM, MAXW) \
     launch_spmm<NB, HALF, BLDS, KS, RM, MAXW>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes, ldb, ldo, relu, \
@@ -1058,6 +1073,18 @@ extern "C" int tcsl_launch_copy(void* stream, void* dst, const void* src, long b
     hipLaunchKernelGGL(tcsl_copy_kernel, dim3(256 * 16), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), bytes / 16);
     return static_cast<int>(hipGetLastError());
+}
+
+// The slab part of the static workspace on the current device: its address and size in bytes.
+// Asks the runtime for the array's address on the first call on a device; allocates nothing.
+extern "C" int tcsl_static_workspace(void** slabs, long* bytes)
+{
+    DeviceArrays a;
+    if (const int rc = device_arrays(&a))
+        return rc;
+    *slabs = a.scratch + kScratchCounterBytes;
+    *bytes = static_cast<long>(kScratchSlabBytes);
+    return 0;
 }
 
 // 1 and *id = the capture's id while `stream` is recording into a graph, 0 while it is not,

@@ -31,6 +31,7 @@ EXPORTED_SYMBOLS = (
     "InitSparseMatrixA_API",
     "InitSparseMatrixA_API_NoReorder",
     "SpMM_SplitK_API",
+    "SpMM_SplitK_API_StaticWorkspace",
     "GenSparseMatrixBinFile",
     "SpMM_FreeHost",
     "SpMM_GetErrorString",
@@ -108,6 +109,8 @@ def load_library():
     lib.InitSparseMatrixA_API_NoReorder.argtypes = lib.InitSparseMatrixA_API.argtypes
     lib.SpMM_SplitK_API.restype = ctypes.c_int
     lib.SpMM_SplitK_API.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_int]
+    lib.SpMM_SplitK_API_StaticWorkspace.restype = ctypes.c_int
+    lib.SpMM_SplitK_API_StaticWorkspace.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int] * 4
     lib.GenSparseMatrixBinFile.restype = ctypes.c_int
     lib.GenSparseMatrixBinFile.argtypes = [ctypes.c_char_p, ctypes.c_int, ctypes.c_int, ctypes.c_char_p,
                                            ctypes.c_char_p, ctypes.c_char_p]
@@ -235,6 +238,18 @@ def SpMM_SplitK_API(stream, A, Compressed_A, TileOffsets, B, C, M_Global, N_Glob
                              _ptr(Reduction_Workspace), Split_K)
     if rc != 0:
         raise SpMMError("SpMM_SplitK_API", rc, lib.SpMM_GetErrorString(rc).decode())
+    return rc
+
+
+def SpMM_SplitK_API_StaticWorkspace(stream, A, Compressed_A, TileOffsets, B, C, M_Global, N_Global, K_Global, Split_K):
+    """SpMM_SplitK_API on the library's static workspace (allocates nothing; Split_K*M*N*2 <= 32 MiB)."""
+    lib = load_library()
+    if stream is not None and not isinstance(stream, int):
+        stream = stream.cuda_stream
+    rc = lib.SpMM_SplitK_API_StaticWorkspace(ctypes.c_void_p(stream) if stream else None, _ptr(A), _ptr(Compressed_A),
+                                             _ptr(TileOffsets), _ptr(B), _ptr(C), M_Global, N_Global, K_Global, Split_K)
+    if rc != 0:
+        raise SpMMError("SpMM_SplitK_API_StaticWorkspace", rc, lib.SpMM_GetErrorString(rc).decode())
     return rc
 
 

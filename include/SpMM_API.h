@@ -101,6 +101,24 @@ SPMM_EXPORT int SpMM_SplitK_API(void* stream, const void* A, const void* Compres
                     void* C, int M_Global, int N_Global, int K_Global, void* Reduction_Workspace, int Split_K);
 
 /*
+ * SpMM_SplitK_API for callers that must not allocate and have no workspace to pass: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the
+ * reference, whose caller allocates 128 MiB once (third_party/ft.patch:2762-2765).  Same
+ * arguments without Reduction_Workspace, same checks, same results bit for bit: the slabs of
+ * partial sums and the arrival counters of the in-launch reduction live in a static device array
+ * of 32 MiB + 16 KiB that every GPU the library runs on holds until the process ends.  The call
+ * allocates and frees nothing (neither does SpMM_SplitK_API itself; here the caller need not
+ * either).  hipErrorInvalidValue, with a message, when Split_K*M*N*2 exceeds 32 MiB (every
+ * OPT-30B/66B/175B layer shape fits with the planner's Split_K up to 64 tokens).  All calls on a
+ * GPU share that one array: calls of this entry point that may overlap on one GPU (different
+ * streams, concurrent graph launches) race and must be ordered by the caller; calls on one
+ * stream are ordered already.
+ */
+SPMM_EXPORT int SpMM_SplitK_API_StaticWorkspace(void* stream, const void* A, const void* Compressed_A,
+                                                const int* TileOffsets, const void* B, void* C, int M_Global,
+                                                int N_Global, int K_Global, int Split_K);
+
+/*
  * SpMM_SplitK_API for row-major operands: B[k*N + n] (K x N) and C[m*N + n] (M x N), with
  * the split-K slabs in the same M x N layout.  This is the convention of this checkout's
  * kernel (csrc/SpMM_Kernel.cuh:372-374 for B, :731-734 for the output; its benchmark passes a
