@@ -83,10 +83,16 @@ bool complete_plan(int N, int K, int split_k, bool row_major, LaunchPlan& p)
         lds += static_cast<long>(p.waves) * N * 128;  // one tile's activations per wave, being transposed
     }
     if (p.mode == 0) {
-        if (p.stage_b) {
+        if (p.stage_b == 1) {  // the batch's whole slice, up to 16 tokens
             if (nb != 1)
                 return false;
             lds += tiles * (N == 8 ? 8 : 16) * 128;
+        } else if (p.stage_b == 2) {  // one tile at a time through two buffers, 32 and 64 tokens
+            if (row_major || !((N == 32 && (p.waves == 4 || p.waves == 8)) || (N == 64 && p.waves == 4)))
+                return false;
+            lds += 2L * N * 128;
+        } else if (p.stage_b != 0) {
+            return false;
         }
     } else if (p.mode == 1) {
         if (p.stage_b)

@@ -305,9 +305,17 @@ __device__ __forceinline__ void fused_reduction_tail(const _Float16* __restrict_
 // ROWMAJ = B is [K][N] and the output [M][N].  HALF = N is 8 (the upper eight columns of the single block are computed on duplicates
 // and dropped); BLDS = the batch's activation slice is staged in LDS; MAXW bounds W and
 // with it the registers a wave may use.
-// Dynamic LDS: W tiles of 16 KiB, then tokens * 128 bytes times tiles_per_batch (BLDS) or times W
-// (ROWMAJ); with KSPLIT at least 8 * W * NB KiB in all (the waves' accumulators meet there).
-template<int NB, bool HALF, bool BLDS, bool KSPLIT, bool ROWMAJ, int MAXW>
+// BSW > 0 (row-sharing layout, 32 or 64 tokens): the W = BSW waves of the workgroup walk their tile
+// rows in step and share each 64-column activation tile through LDS: every wave fetches its
+// 1/BSW of the tile's tokens with full-line loads (together with its own words of that tile,
+// two tiles ahead), writes it into one of two tile buffers, and after one barrier per tile all
+// read their MFMA operands from there.  That cuts the activation bytes a compute unit pulls
+// through its vector memory path by BSW, which is what bounds 32 and 64 tokens otherwise (the
+// fragments of one tile are 4 or 8 KiB against 6.5 KiB of weight words, and they cost about half
+// as much per byte although they come from the L2).
+// Dynamic LDS: W tiles of 16 KiB, then tokens * 128 bytes times tiles_per_batch (BLDS), times W
+// (ROWMAJ) or times two (BSW); with KSPLIT at least 8 * W * NB KiB in all (the waves' accumulators meet there).
+template<int NB, bool HALF, bool BLDS, bool KSPLIT, bool ROWMAJ, int MAXW, int BSW = 0>
 __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __restrict__ offsets,
                                                                 const u32x4* __restrict__ items,
                                                                 const _Float16* __restrict__ B,
@@ -326,11 +334,16 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
     constexpr int D = kRing;
     constexpr int NTOK = HALF ? 8 : NB * 16;      // tokens
     // activation loads per issue: two fragments per column block, or (ROWMAJ) the tile's
-    // 64 x N block as 1 KiB pieces
-    constexpr int BL = BLDS ? 0 : (ROWMAJ ? NTOK / 8 : 2 * NB);
+    // 64 x N block as 1 KiB pieces, or (BSW) this wave's share of the tile's tokens, eight
+    // tokens' 128-byte lines per load
+    constexpr int kShareTokens = BSW > 0 ? NTOK / BSW : 0;  // tokens this wave fetches per tile
+    constexpr int BL = BLDS ? 0 : BSW > 0 ? (kShareTokens + 7) / 8 : (ROWMAJ ? NTOK / 8 : 2 * NB);
 
     static_assert(!(KSPLIT && BLDS), "a workgroup that splits K shares no activation slice");
     static_assert(!(ROWMAJ && BLDS), "row-major activations are not staged");
+    static_assert(BSW == 0 || (!KSPLIT && !BLDS && !ROWMAJ && !HALF && NB >= 2 && NTOK % BSW == 0 && BSW <= MAXW),
+                  "activation tiles are streamed through LDS in the row-sharing layout only");
+
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // uniform, and known to be
     // grid: x = group of tile rows (one tile row in the K-splitting layout), y = split-K batch
@@ -414,7 +427,9 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         kb0 = b0;
         kb1 = b1;
     }
-    const int ntile = active ? kb1 - kb0 : 0;  // tiles of this wave
+    // tiles of this wave (BSW: a wave past the last tile row walks along with empty tiles, for its
+    // share of the activation tiles and for the barriers)
+    const int ntile = active || BSW > 0 ? kb1 - kb0 : 0;
     // Activations in LDS, per tile [token][8 granules of 16 B at position g ^ (token & 7)]: the
     // batch's slice, staged once and shared (BLDS), or (ROWMAJ) a one-tile buffer per wave in
     // which the tile's k-major block is turned into token-major MFMA operands.
@@ -425,7 +440,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
     const int* toff = offsets + (size_t)(active ? rt : 0) * nkb + kb0;
     int wbase = 0;
     if (!KSPLIT)
-        wreg = toff[lane <= ntile ? lane : ntile];
+        wreg = active ? toff[lane <= ntile ? lane : ntile] : 0;
 
     if (BLDS) {
         const int ngran = (kb1 - kb0) * NTOK * 8;  // the whole batch, whatever this wave's own share
@@ -439,15 +454,15 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         clear_tile(tile, lane);
     if (BLDS)
         __syncthreads();  // the only barrier: every wave of the workgroup reaches it
-    if (!KSPLIT && !active && !arrivals)
+    if (!KSPLIT && !active && !arrivals && BSW == 0)
         return;  // (with the fused reduction every wave has to reach the barriers at the end)
     const bool clamp = relu && !arrivals;  // partial sums are never clamped
 
-    auto tile_range = [&](int i, int& begin, int& end) {  // 0 <= i < ntile
+    auto tile_range = [&](int i, int& begin, int& end) __attribute__((always_inline)) {  // 0 <= i < ntile
         if (i + 1 - wbase >= kWave) {  // slide the window (more than 63 tiles per wave only)
             wbase = i;
             const int idx = i + lane;
-            wreg = toff[idx <= ntile ? idx : ntile];
+            wreg = active ? toff[idx <= ntile ? idx : ntile] : 0;
             settle(wreg);  // makes the compiler wait for this load here, on the rare path, not at the join below
         }
         begin = __builtin_amdgcn_readlane(wreg, i - wbase);
@@ -487,6 +502,22 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         for (int s = 0; s < 2; s++)
             b_off[c][s] = tok * 128 + (((s * 4 + q) ^ (tok & 7)) << 4);
     }
+    // BSW: load i of this wave's share of a tile covers tokens share0 + 8 i + (lane >> 3), lane & 7
+    // being the 16-byte granule of the token's 128-byte line; lanes beyond the share (a share of
+    // four tokens fills half a load) repeat a token and write nothing.
+    const _Float16* sh_ptr[BL > 0 ? BL : 1];
+    int sh_off[BL > 0 ? BL : 1];
+    bool sh_ok[BL > 0 ? BL : 1];
+    if (BSW > 0) {
+#pragma unroll
+        for (int i = 0; i < BL; i++) {
+            const int t = 8 * i + (lane >> 3);
+            sh_ok[i] = t < kShareTokens;
+            const int tok = wave * kShareTokens + t % (kShareTokens > 0 ? kShareTokens : 1);
+            sh_ptr[i] = B + (size_t)tok * ldb + (size_t)kb0 * kTileCols + (lane & 7) * 8;
+            sh_off[i] = tok * 128 + (((lane & 7) ^ (tok & 7)) << 4);
+        }
+    }
     // Per-lane byte offsets of the word loads: chunk u sits at lane*16 + u*1024 and the
     // instruction's immediate offset reaches 4095.
     const int voff_lo = lane * 16, voff_hi = lane * 16 + 4096, voff_top = lane * 16 + 8192;
@@ -503,7 +534,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
     // holds, which on small tiles (90 % sparsity and up) is 5 to 14 % of the time.  So a
     // workgroup (or, in the row-sharing layout, a wave) picks by its own run's density
     // (`segments`, set where the density is read).
-    auto stream_run = [&](auto vpl_c) {
+    auto stream_run = [&](auto vpl_c) __attribute__((always_inline)) {
         constexpr int VPL = decltype(vpl_c)::value;
         constexpr int L = VPL + BL;        // loads per issue: word loads (+ activation loads)
         constexpr int kSeg = VPL * kWave;  // vectors per segment
@@ -526,7 +557,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         struct Cur {
             int tile, off;
         };
-        auto make_seg = [&](Cur c, Seg& s, Cur& nxt) {
+        auto make_seg = [&](Cur c, Seg& s, Cur& nxt) __attribute__((always_inline)) {
             if (c.tile >= ntile) {
                 s = Seg{ntile, 0, 0, true, true};
                 nxt = c;
@@ -548,7 +579,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         Seg held[D] = {};
 
         // Always exactly L loads, whatever the segment holds, so the wait counts are static.
-        auto issue = [&](int slot, const Seg& s) {
+        auto issue = [&](int slot, const Seg& s) __attribute__((always_inline)) {
             if (held[slot ^ 1].n + s.n > flight)
                 wait_loads<0>();
             const bool live = s.tile < ntile;
@@ -559,7 +590,11 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
             // so behind the weight loads they would hold their slots for a full HBM round trip (1-3 %).
             if (!BLDS) {
                 const int bt = live ? s.tile : ntile - 1;
-                if (ROWMAJ) {
+                if (BSW > 0) {
+    #pragma unroll
+                    for (int h = 0; h < BL; h++)
+                        bfrag[slot][h] = load_activations(sh_ptr[h] + bt * kTileCols);
+                } else if (ROWMAJ) {
                     // B[k][n]: the tile's 64 x N block is contiguous; piece h = bytes [1024 h, 1024 h + 1024)
                     const _Float16* blk = B + (size_t)(kb0 + bt) * (kTileCols * NTOK);
     #pragma unroll
@@ -587,7 +622,7 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         // Waits for every load of `slot` (at most Y younger ones may stay in flight) and keeps the
         // slot's registers live up to that point, so none of them can be reused while a load into
         // it is still on its way.
-        auto land = [&](int slot, auto younger) {
+        auto land = [&](int slot, auto younger) __attribute__((always_inline)) {
             constexpr int Y = decltype(younger)::value;
             wait_loads<Y>();
             static_for<VPL>([&](auto uc) { pin(regs[slot][decltype(uc)::value]); });
@@ -601,8 +636,24 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         // Y = loads issued after this slot's that may stay in flight.  The slot's loads were issued
         // a whole tile ago, so waiting for all of them up front costs nothing in steady state and
         // keeps one unconditional wait on every path through the loop.
-        auto consume = [&](int slot, const Seg& s, auto younger) {
+        auto consume = [&](int slot, const Seg& s, auto younger) __attribute__((always_inline)) {
             land(slot, younger);
+            if (BSW > 0 && s.tile < ntile) {
+                // This wave's share of the tile's activations goes into the tile's buffer with the
+                // tile's first segment; one barrier per tile, ahead of its last segment (every tile
+                // has one, an empty tile too: the other waves count on it).  Before the barrier every
+                // wave has written its share and has finished reading the previous tile's activations
+                // from the other buffer, so after it this tile's buffer is complete and the other one
+                // may be written for the next tile.
+                if (s.first) {
+    #pragma unroll
+                    for (int h = 0; h < BL; h++)
+                        if (sh_ok[h])
+                            *reinterpret_cast<half8*>(bslice + (s.tile & 1) * (NTOK * 128) + sh_off[h]) = bfrag[slot][h];
+                }
+                if (s.last)
+                    __syncthreads();
+            }
             if (s.n == 0)
                 return;  // empty tile or past the end
             uint32_t kept[VPL][4];  // the scatter's LDS addresses, for the un-scatter
@@ -635,8 +686,8 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
             if (!s.last)
                 return;  // more segments of this tile follow
             half8 bf[NB][2];
-            if (BLDS || ROWMAJ) {
-                const uint8_t* bt = bslice + (BLDS ? (size_t)s.tile * (NTOK * 128) : 0);
+            if (BLDS || ROWMAJ || BSW > 0) {
+                const uint8_t* bt = bslice + (BLDS ? (size_t)s.tile * (NTOK * 128) : BSW > 0 ? (s.tile & 1) * (NTOK * 128) : 0);
                 if (ROWMAJ) {
                     // lane l of piece h holds tokens n0 .. n0+7 of row k, (k, n0) = divmod(512 h + 8 l, N);
                     // element (k, n) goes to byte n*128 + (((k >> 3) ^ (n & 7)) << 4) + 2*(k & 7), n & 7 = j
@@ -956,14 +1007,16 @@ int device_arrays(DeviceArrays* out)
     return 0;
 }
 
-template<int NB, bool HALF, bool BLDS, bool KSPLIT, bool ROWMAJ, int MAXW>
+template<int NB, bool HALF, bool BLDS, bool KSPLIT, bool ROWMAJ, int MAXW, int BSW = 0>
 int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const void* B, void* out, int M, int N,
                 int K, int split_k, int waves, unsigned lds_bytes, int ldb, int ldo, int relu, void* fused_out,
                 int ldc, unsigned int* arrivals, int dense_waves)
 {
     if (waves < 1 || waves > MAXW || lds_bytes > kMaxLdsBytes)
         return static_cast<int>(hipErrorInvalidValue);
-    auto kernel = tcsl_spmm_kernel<NB, HALF, BLDS, KSPLIT, ROWMAJ, MAXW>;
+    if (BSW > 0 && waves != BSW)
+        return static_cast<int>(hipErrorInvalidValue);
+    auto kernel = tcsl_spmm_kernel<NB, HALF, BLDS, KSPLIT, ROWMAJ, MAXW, BSW>;
     // more than 64 KiB of dynamic LDS has to be allowed once per kernel (per device, re-armed lazily)
     static std::atomic<int> armed_device{-1};
     int dev = 0;
@@ -995,8 +1048,10 @@ int launch_spmm(hipStream_t stream, const void* items, const int* offsets, const
 // Launchers called by the host logic.  Shapes are validated by the caller; all
 // pointers are device memory; everything is asynchronous on `stream`.
 
-// mode 0: the W waves of a workgroup take W consecutive tile rows of one batch (and, with
-//         stage_b != 0 and N <= 16, share the batch's activation slice in LDS);
+// mode 0: the W waves of a workgroup take W consecutive tile rows of one batch; with stage_b = 1
+//         (N <= 16) they share the batch's activation slice, staged once in LDS; with stage_b = 2
+//         (N = 32: 4 or 8 waves, N = 64: 4 waves) they walk the batch in step and share each
+//         activation tile through LDS;
 // mode 1: the W waves of a workgroup split the batch of one tile row among themselves and
 //         add their results up in LDS (stage_b must be 0).
 // row_major: B is [K][N] and the output [M][N] instead of [N][K] and [N][M] (stage_b must be 0).
@@ -1017,7 +1072,11 @@ extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offs
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (mode != 0 && mode != 1)
         return static_cast<int>(hipErrorInvalidValue);
-    if (stage_b && (mode == 1 || row_major || N > 16))
+    if (stage_b == 1 && (mode == 1 || row_major || N > 16))
+        return static_cast<int>(hipErrorInvalidValue);
+    if (stage_b == 2 && (mode == 1 || row_major || !((N == 32 && (waves == 4 || waves == 8)) || (N == 64 && waves == 4))))
+        return static_cast<int>(hipErrorInvalidValue);
+    if (stage_b < 0 || stage_b > 2)
         return static_cast<int>(hipErrorInvalidValue);
     unsigned int* arrivals = nullptr;
     if (fuse_page >= 0) {
@@ -1031,8 +1090,8 @@ extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offs
         arrivals = fuse_page == kScratchPage ? reinterpret_cast<unsigned int*>(a.scratch)
                                              : a.arrivals + static_cast<size_t>(fuse_page) * kCountersPerPage;
     }
-#define TCSL_GO(NB, HALF, BLDS, KS, RM, MAXW) \
-    launch_spmm<NB, HALF, BLDS, KS, RM, MAXW>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes, ldb, ldo, relu, \
+#define TCSL_GO(NB, HALF, BLDS, KS, RM, MAXW, ...) \
+    launch_spmm<NB, HALF, BLDS, KS, RM, MAXW, ##__VA_ARGS__>(s, items, offsets, B, out, M, N, K, split_k, waves, lds_bytes, ldb, ldo, relu, \
                                               fused_out, ldc, arrivals, dense_waves)
 #define TCSL_PICK(NB, HALF, MAXW)                                                                     \
     (row_major ? (mode ? TCSL_GO(NB, HALF, false, true, true, MAXW) : TCSL_GO(NB, HALF, false, false, true, MAXW)) \
@@ -1043,8 +1102,12 @@ extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offs
         case 16:
             return stage_b ? TCSL_GO(1, false, true, false, false, 8) : TCSL_PICK(1, false, 8);
         case 32:
+            if (stage_b == 2)
+                return waves == 8 ? TCSL_GO(2, false, false, false, false, 8, 8) : TCSL_GO(2, false, false, false, false, 8, 4);
             return TCSL_PICK(2, false, 8);
         case 64:
+            if (stage_b == 2)
+                return TCSL_GO(4, false, false, false, false, 4, 4);
             return TCSL_PICK(4, false, 4);
         default:
             return static_cast<int>(hipErrorInvalidValue);

@@ -35,6 +35,10 @@ def candidate_plans(N, tiles_k):
                 plans += [(S, 0, w, 1) for w in (5, 6, 7, 8)]
             else:
                 plans += [(S, 0, w, 0) for w in (1, 2, 4)]
+    if N >= 32:  # the waves share each activation tile through LDS
+        for S in (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 14, 16, 20, 24, 28, 32):
+            if S <= tiles_k:
+                plans += [(S, 0, w, 2) for w in ((4, 8) if N == 32 else (4,))]
     return plans
 
 

@@ -226,7 +226,9 @@ SPMM_EXPORT int SpMM_SuggestSplitK(int M_Global, int N_Global, int K_Global);
 /*
  * The launch shape SpMM_SplitK_API uses for (M, N, K, Split_K):
  *   Mode 0  the Waves waves of a workgroup take consecutive 128-row tile rows of one
- *           split-K batch (StageB: they share the batch's activation slice in LDS);
+ *           split-K batch (StageB = 1, up to 16 tokens: they share the batch's activation slice,
+ *           staged once in LDS; StageB = 2, 32 tokens with 4 or 8 waves and 64 tokens with 4:
+ *           they walk the batch in step and share each 64-column activation tile through LDS);
  *   Mode 1  the Waves waves of a workgroup split the batch of one tile row among
  *           themselves and add their accumulators up in LDS.
  * Any output pointer may be NULL.  EstimatedUs is the cost model's figure for the whole
@@ -240,7 +242,8 @@ SPMM_EXPORT int SpMM_PlanLaunch(int M_Global, int N_Global, int K_Global, int Sp
  * SpMM_SplitK_API with the launch shape given by the caller instead of the planner
  * (for tuning a table of plans on the target machine, and for tests).  Returns
  * hipErrorInvalidValue when the shape does not fit (Waves above 8, or 4 for N = 64;
- * StageB with Mode 1, N > 16 or RowMajor; more than 160 KiB of LDS).  RowMajor != 0 selects
+ * StageB with Mode 1 or RowMajor, StageB = 1 with N > 16, StageB = 2 outside the shapes above;
+ * more than 160 KiB of LDS).  RowMajor != 0 selects
  * the operand layout of SpMM_SplitK_API_RowMajor; Flags as for SpMM_SplitK_API_Strided (no
  * clamp with row-major operands).  No counterpart in the reference.
  */

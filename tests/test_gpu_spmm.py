@@ -888,3 +888,49 @@ def test_graph_replay_beside_eager_calls_on_the_capture_stream(spmm):
         torch.cuda.synchronize()
         assert np.array_equal(gC.cpu().numpy().view(np.uint16), want), f"replay {rep}"
         assert np.array_equal(eC.cpu().numpy().view(np.uint16), want), f"eager beside replay {rep}"
+
+
+@pytest.mark.parametrize("M,K,N,split_k,waves,sparsity", [
+    (1024, 1024, 32, 4, 4, 0.8),
+    (1024, 1024, 32, 2, 8, 0.8),
+    (1024, 1024, 64, 2, 4, 0.8),
+    (1152, 1536, 64, 3, 4, 0.8),     # nine tile rows: the last workgroup has three waves without rows
+    (640, 2048, 32, 1, 8, 0.8),      # five tile rows over eight waves, no split: the kernel writes C itself
+    (512, 1024, 64, 2, 4, 0.5),      # tiles of several segments (the image is cleared, not un-scattered)
+    (512, 1024, 32, 2, 4, 0.3),
+    (1024, 2048, 64, 4, 4, 0.95),    # short segments, some waves on sparser rows than others
+    (512, 64 * 70, 32, 1, 4, 0.9),   # more than 63 tiles per wave: the offsets window slides
+])
+def test_shared_activation_tiles_through_lds(spmm, oracle, M, K, N, split_k, waves, sparsity):
+    """Row-sharing launch whose waves walk their tile rows in step and share each activation tile
+    through LDS (StageB = 2), 32 and 64 tokens: against the oracle, with the second-kernel and the
+    in-launch reduction, and with empty tiles and rows of different density in one workgroup."""
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    A = spmm.synth_weights(M, K, sparsity, False, seed=M + K + N + waves)
+    A[128:256, :] = spmm.synth_weights(128, K, min(0.99, sparsity + 0.15), False, seed=3)   # a sparser tile row
+    A[0:128, 64:192] = 0                                                                   # two empty tiles
+    if M >= 512:
+        A[384:512, :] = 0                                                                  # a whole empty tile row
+    B = spmm.synth_activations(N, K, seed=M + 1)
+    items, offsets = spmm.InitSparseMatrixA_API(A)
+    ref = oracle.gemm_f32(A, B)
+    d_items = torch.from_numpy(items.view(np.int32).copy()).to(dev)
+    d_offs = torch.from_numpy(offsets.copy()).to(dev)
+    d_B = torch.from_numpy(B.view(np.int16).copy()).to(dev)
+    for flags in (0, spmm.SPMM_FLAG_SEPARATE_REDUCTION):
+        d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device=dev)
+        d_W = torch.full((split_k, N, M), float("nan"), dtype=torch.float16, device=dev) if split_k > 1 else None
+        print(f"[gpu case] shared activation tiles M={M} K={K} N={N} split_k={split_k} waves={waves} flags={flags}", flush=True)
+        spmm.SpMM_SplitK_API_Planned(torch.cuda.current_stream(), d_items, d_offs, d_B, d_C, M, N, K, d_W, split_k, 0,
+                                     waves, 2, 0, flags)
+        torch.cuda.synchronize()
+        assert_close(d_C.cpu().numpy(), ref)
+
+
+def test_shared_activation_tiles_rejects_other_shapes(spmm):
+    torch = _torch()
+    z = torch.zeros(1024, dtype=torch.int32, device="cuda:0")
+    for (N, mode, waves, row_major) in [(16, 0, 4, 0), (32, 0, 2, 0), (64, 0, 2, 0), (32, 1, 4, 0), (64, 0, 4, 1), (8, 0, 8, 0)]:
+        with pytest.raises(spmm.SpMMError):
+            spmm.SpMM_SplitK_API_Planned(None, z, z, z, z, 1024, N, 1024, z, 1, mode, waves, 2, row_major)

@@ -162,8 +162,13 @@ def test_planner_gives_runnable_plans(spmm):
                 assert 1 <= p["waves"] <= (8 if N <= 32 else 4)
                 assert p["lds_bytes"] <= 160 * 1024
                 assert p["lds_bytes"] >= p["waves"] * 16384
-                if p["stage_b"]:
+                if p["stage_b"] == 1:    # the batch's slice staged once
                     assert p["mode"] == 0 and N <= 16
+                elif p["stage_b"] == 2:  # tile by tile through two buffers
+                    assert p["mode"] == 0 and ((N == 32 and p["waves"] in (4, 8)) or (N == 64 and p["waves"] == 4))
+                    assert p["lds_bytes"] == p["waves"] * 16384 + 2 * N * 128
+                else:
+                    assert p["stage_b"] == 0
                 assert 0 < p["estimated_us"] < 1e6
     with pytest.raises(spmm.SpMMError):
         spmm.SpMM_PlanLaunch(1000, 16, 1024, 1)
