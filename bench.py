@@ -15,9 +15,10 @@ Prints ONE JSON line:
   value           effective TFLOPS, 2*M*N*K / step time (whole call)
   hbm_gbps        compressed-weight bytes / step time
   roofline        the main kernel alone: algorithmic bytes (16 * TileOffsets[last])
-                  / its average duration, from two HIP events recorded on the launch
-                  stream around K back-to-back launches of it (median of --repeats such
-                  blocks), against the 8 TB/s HBM peak
+                  / its average duration, from HIP events recorded on the launch stream
+                  around blocks of K back-to-back launches of it (--repeats blocks enqueued
+                  without a host synchronisation in between; the median block), against the
+                  8 TB/s HBM peak
   cpu_baseline    the CPU path timed on this host: reference encoder (oracle/_ref,
                   single thread) + fp32-accumulate dense GEMM (oracle, single thread)
   sweep           the benchmark's other configurations, each timed for a fraction of a
@@ -148,6 +149,24 @@ def events_ms(lib, sptr, call, n):
     return ms
 
 
+def chained_events_ms(lib, sptr, call, n, blocks):
+    """`blocks` blocks of n calls enqueued back to back, an event between every two blocks and
+    no host synchronisation in between: the milliseconds of each block, with the stream kept busy
+    throughout (so no block pays the start-up latency of a launch into an idle queue)."""
+    events = [lib.SpMM_EventCreate() for _ in range(blocks + 1)]
+    lib.SpMM_EventRecord(events[0], sptr)
+    k = 0
+    for b in range(blocks):
+        for _ in range(n):
+            call(k)
+            k += 1
+        lib.SpMM_EventRecord(events[b + 1], sptr)
+    ms = [float(lib.SpMM_EventElapsedMs(events[b], events[b + 1])) for b in range(blocks)]
+    for e in events:
+        lib.SpMM_EventDestroy(e)
+    return ms
+
+
 SWEEP = [
     # (label, workload, N, sparsity, row_skewed)
     ("ffn1_n8", "opt30b_ffn1", 8, 0.8, False),
@@ -186,7 +205,7 @@ def sweep(G, lib, torch, dev, sptr, with_stack):
             d_offs = [torch.from_numpy(offsets).to(dev) for _ in range(copies)]
             cache[key] = (a_bytes, copies, d_items, d_offs)
         a_bytes, copies, d_items, d_offs = cache[key]
-        split_k = G.SpMM_SuggestSplitK(M, N, K)
+        split_k = G.SpMM_SuggestSplitK_Bytes(M, N, K, a_bytes // 16)
         d_B = torch.from_numpy(G.synth_activations(N, K, seed=4321).view(np.int16)).to(dev)
         d_C = torch.zeros((N, M), dtype=torch.float16, device=dev)
         d_W = torch.zeros((max(split_k, 1), N, M), dtype=torch.float16, device=dev)
@@ -274,7 +293,7 @@ def main():
     ap.add_argument("--n", type=int, default=None, help="override the token count N")
     ap.add_argument("--sparsity", type=float, default=None)
     ap.add_argument("--skew", action="store_true")
-    ap.add_argument("--split-k", type=int, default=0, help="0 = SpMM_SuggestSplitK")
+    ap.add_argument("--split-k", type=int, default=0, help="0 = SpMM_SuggestSplitK_Bytes")
     ap.add_argument("--copies", type=int, default=0, help="distinct HBM copies of the weight (0 = enough for > 640 MB)")
     ap.add_argument("--no-reorder", action="store_true",
                     help="encode with InitSparseMatrixA_API_NoReorder (the reference's ablation of its bank-aware reordering)")
@@ -309,7 +328,7 @@ def main():
     if args.sparsity is not None:
         sparsity = args.sparsity
     skew = skew or args.skew
-    split_k = args.split_k or G.SpMM_SuggestSplitK(M, N, K)
+    split_k = args.split_k  # 0: chosen below, once the weight's size is known
 
     # ---- synthetic inputs (host), encode (host), upload
     t0 = time.perf_counter()
@@ -320,6 +339,7 @@ def main():
     items, offsets = (G.InitSparseMatrixA_API_NoReorder if args.no_reorder else G.InitSparseMatrixA_API)(A)
     t_encode = time.perf_counter() - t0
     a_bytes = 16 * int(offsets[-1])
+    split_k = split_k or G.SpMM_SuggestSplitK_Bytes(M, N, K, a_bytes // 16)
     copies = args.copies or max(2, -(-640 * 1024 * 1024 // max(a_bytes, 1)))
     copies = min(copies, 64)
 
@@ -392,7 +412,7 @@ def main():
 
     for i in range(200):
         partials(i)
-    kernel_blocks_ms = [events_ms(lib, sptr, partials, args.steps) for _ in range(max(1, args.repeats))]
+    kernel_blocks_ms = chained_events_ms(lib, sptr, partials, args.steps, max(1, args.repeats))
     kernel_ms_avg = float(np.median(kernel_blocks_ms)) / args.steps
     torch.cuda.synchronize()
 

@@ -23,7 +23,7 @@ constexpr int kCUs = 256;
 
 // Fitted constants (microseconds, bytes per microsecond).
 constexpr double kLaunchUs = 1.83;          // fixed cost of the main kernel
-constexpr double kTileBytes = 6558.0;       // one tile at 80 % sparsity
+constexpr double kTileBytes = kTileBytesAt80;  // one tile at 80 % sparsity: what the constants below were fitted on
 constexpr double kChipBytesPerUs = 7.0e6;   // whole-chip stream rate
 constexpr double kCuBytesPerUs = 39.2e3;    // what one compute unit can pull on its own
 constexpr double kWaveTileUs = 0.367;       // a lone wave's turnaround per tile (latency bound)
@@ -48,21 +48,55 @@ int max_waves(int N)
     return N <= 32 ? 8 : 4;  // registers: two waves per SIMD up to N = 32, one at N = 64
 }
 
-// Measured optimum for the layer shapes of OPT-30B and OPT-66B (80 % sparsity):
-// {M, K, N, Split_K, mode, waves, stage_b}.
+// Measured optima for the layer shapes of OPT-30B and OPT-66B, {M, K, N, Split_K, mode, waves,
+// stage_b}: one table per sparsity the benchmark names.  A caller that knows the weight's bytes
+// gets its Split_K from the table of the nearest density; a call, which knows only (M, N, K,
+// Split_K), takes the launch shape of whichever table holds that Split_K for the shape (80 %
+// first), so the Split_K that a converter stored carries the choice to the run.
 struct Tuned {
     int M, K, N, split_k, mode, waves, stage_b;
 };
-constexpr Tuned kTuned[] = {
+constexpr Tuned kTuned80[] = {
 #include "tuned_plans.inc"
 };
+constexpr Tuned kTuned70[] = {
+#include "tuned_plans_70.inc"
+};
+constexpr Tuned kTuned90[] = {
+#include "tuned_plans_90.inc"
+};
 
-const Tuned* find_tuned(int M, int N, int K)
+// 0: the 80 % table (also for an unknown density), 1: 70 %, 2: 90 %; boundaries at 75 % and 85 % sparsity
+int density_table(double tile_bytes)
 {
-    for (const Tuned& t : kTuned)
-        if (t.M == M && t.K == K && t.N == N)
+    if (!(tile_bytes > 0.0))
+        return 0;
+    return tile_bytes > 1.25 * kTileBytes ? 1 : tile_bytes < 0.75 * kTileBytes ? 2 : 0;
+}
+
+template<int Rows>
+const Tuned* find_in(const Tuned (&table)[Rows], int M, int N, int K, int split_k)
+{
+    for (const Tuned& t : table)
+        if (t.M == M && t.K == K && t.N == N && (split_k == 0 || t.split_k == split_k))
             return &t;
     return nullptr;
+}
+
+// split_k == 0: any.  which = 0, 1, 2 as density_table(); -1: every table, the 80 % one first, then 70 %, then 90 %
+const Tuned* find_tuned(int M, int N, int K, int split_k, int which)
+{
+    const Tuned* t = nullptr;
+    // (The 90 % table comes last: a K-splitting launch of a sparse weight picks its number of
+    // streaming waves per tile row in the kernel, so that table's wave counts say little, while
+    // the denser tables' counts are what dense tile rows run with.)
+    if (which == 0 || which < 0)
+        t = find_in(kTuned80, M, N, K, split_k);
+    if (!t && (which == 1 || which < 0))
+        t = find_in(kTuned70, M, N, K, split_k);
+    if (!t && (which == 2 || which < 0))
+        t = find_in(kTuned90, M, N, K, split_k);
+    return t;
 }
 
 }  // namespace
@@ -109,8 +143,10 @@ bool complete_plan(int N, int K, int split_k, bool row_major, LaunchPlan& p)
     return true;
 }
 
-double plan_cost_us(int M, int N, int K, int split_k, const LaunchPlan& p)
+double plan_cost_us(int M, int N, int K, int split_k, const LaunchPlan& p, double tile_bytes)
 {
+    if (!(tile_bytes > 0.0))
+        tile_bytes = kTileBytes;
     const long row_tiles = M / kTileRows;
     const long nkb = K / kTileCols;
     const int nb = column_blocks(N);
@@ -130,8 +166,8 @@ double plan_cost_us(int M, int N, int K, int split_k, const LaunchPlan& p)
     if (fit < 1 || (p.mode == 1 && N <= 32))
         fit = 1;  // (a K-splitting plan is launched with eight waves: one workgroup per compute unit)
     const long slots = kCUs * fit;
-    const double tau_chip = kTileBytes / kChipBytesPerUs;
-    const double tau_cu = kTileBytes / kCuBytesPerUs;
+    const double tau_chip = tile_bytes / kChipBytesPerUs;
+    const double tau_cu = tile_bytes / kCuBytesPerUs;
     const double tau_wave = kWaveTileUs + kMfmaTileUs * nb;
     double total = kLaunchUs;
     for (long left = wgs; left > 0;) {
@@ -153,13 +189,14 @@ double plan_cost_us(int M, int N, int K, int split_k, const LaunchPlan& p)
     return total;
 }
 
-LaunchPlan plan_launch(int M, int N, int K, int split_k, bool row_major, double* cost_us)
+LaunchPlan plan_launch(int M, int N, int K, int split_k, bool row_major, double* cost_us, double tile_bytes)
 {
-    if (const Tuned* t = find_tuned(M, N, K)) {
+    // a measured optimum with this Split_K: of the weight's own density if the caller gave it, else of any
+    if (const Tuned* t = find_tuned(M, N, K, split_k, tile_bytes > 0.0 ? density_table(tile_bytes) : -1)) {
         LaunchPlan p{t->mode, t->waves, t->stage_b, 0};
-        if (t->split_k == split_k && complete_plan(N, K, split_k, row_major, p)) {
+        if (complete_plan(N, K, split_k, row_major, p)) {
             if (cost_us)
-                *cost_us = plan_cost_us(M, N, K, split_k, p);
+                *cost_us = plan_cost_us(M, N, K, split_k, p, tile_bytes);
             return p;
         }
     }
@@ -181,7 +218,7 @@ LaunchPlan plan_launch(int M, int N, int K, int split_k, bool row_major, double*
                 LaunchPlan p{mode, w, stage, 0};
                 if (!complete_plan(N, K, split_k, row_major, p))
                     continue;
-                const double c = plan_cost_us(M, N, K, split_k, p);
+                const double c = plan_cost_us(M, N, K, split_k, p, tile_bytes);
                 if (best_cost < 0 || c < best_cost) {
                     best = p;
                     best_cost = c;
@@ -192,9 +229,9 @@ LaunchPlan plan_launch(int M, int N, int K, int split_k, bool row_major, double*
     return best;
 }
 
-int suggest_split_k(int M, int N, int K, LaunchPlan* plan)
+int suggest_split_k(int M, int N, int K, LaunchPlan* plan, double tile_bytes)
 {
-    if (const Tuned* t = find_tuned(M, N, K)) {
+    if (const Tuned* t = find_tuned(M, N, K, 0, density_table(tile_bytes))) {
         LaunchPlan p{t->mode, t->waves, t->stage_b, 0};
         if (complete_plan(N, K, t->split_k, false, p)) {
             if (plan)
@@ -211,7 +248,7 @@ int suggest_split_k(int M, int N, int K, LaunchPlan* plan)
         if (s > 1 && tiles * (s - 1) >= nkb)
             continue;  // a split that leaves the last batch empty
         double c = 0.0;
-        const LaunchPlan p = plan_launch(M, N, K, static_cast<int>(s), false, &c);
+        const LaunchPlan p = plan_launch(M, N, K, static_cast<int>(s), false, &c, tile_bytes);
         if (best_cost < 0 || c < best_cost - 1e-9) {
             best = static_cast<int>(s);
             best_cost = c;

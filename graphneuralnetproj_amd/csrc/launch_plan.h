@@ -18,13 +18,16 @@ struct LaunchPlan {
 bool complete_plan(int N, int K, int split_k, bool row_major, LaunchPlan& p);
 
 // Estimated time in microseconds of SpMM_SplitK_API (main kernel + reduction) with this plan.
-double plan_cost_us(int M, int N, int K, int split_k, const LaunchPlan& p);
+// tile_bytes: average compressed bytes per 128 x 64 tile of the weight (16 * vectors / tiles);
+// 0 = not known, taken as 80 % sparsity.
+constexpr double kTileBytesAt80 = 6558.0;
+double plan_cost_us(int M, int N, int K, int split_k, const LaunchPlan& p, double tile_bytes = 0.0);
 
 // Best plan for a given Split_K; *cost_us (optional) receives its estimate.
 // row_major: B is [K][N] and C [M][N]; such calls cannot stage the activation slice.
-LaunchPlan plan_launch(int M, int N, int K, int split_k, bool row_major, double* cost_us);
+LaunchPlan plan_launch(int M, int N, int K, int split_k, bool row_major, double* cost_us, double tile_bytes = 0.0);
 
 // Best Split_K in 1..32 (with its plan) for the shape.
-int suggest_split_k(int M, int N, int K, LaunchPlan* plan);
+int suggest_split_k(int M, int N, int K, LaunchPlan* plan, double tile_bytes = 0.0);
 
 }  // namespace tcsl

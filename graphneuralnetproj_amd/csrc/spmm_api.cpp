@@ -412,6 +412,14 @@ extern "C" int SpMM_SuggestSplitK(int M, int N, int K)
                                  K - K % tcsl::kTileCols > 0 ? K - K % tcsl::kTileCols : tcsl::kTileCols, nullptr);
 }
 
+extern "C" int SpMM_SuggestSplitK_Bytes(int M, int N, int K, long Vectors)
+{
+    if (M <= 0 || K <= 0 || (N != 8 && N != 16 && N != 32 && N != 64) || M % tcsl::kTileRows != 0 || K % tcsl::kTileCols != 0)
+        return 1;
+    const double tiles = static_cast<double>(M / tcsl::kTileRows) * (K / tcsl::kTileCols);
+    return tcsl::suggest_split_k(M, N, K, nullptr, Vectors > 0 ? 16.0 * static_cast<double>(Vectors) / tiles : 0.0);
+}
+
 extern "C" void SpMM_SynthWeights(uint16_t* A_h, int M, int K, double sparsity, int row_skewed, uint64_t seed)
 {
     tcsl::synth_weights(A_h, M, K, sparsity, row_skewed, seed);

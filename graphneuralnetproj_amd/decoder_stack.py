@@ -56,7 +56,7 @@ def build_layer(G, torch, dev, h, N, sparsity, seed, keep_dense=False, weight_sc
             A = (A.astype(np.float32) * weight_scale).astype(np.float16)
         items, offsets = G.InitSparseMatrixA_API(A)
         mats[name] = (torch.from_numpy(items.view(np.int32)).to(dev), torch.from_numpy(offsets).to(dev), M, K,
-                      G.SpMM_SuggestSplitK(M, N, K))
+                      G.SpMM_SuggestSplitK_Bytes(M, N, K, int(offsets[-1])))
         if keep_dense:
             dense[name] = A
     return Layer(mats), dense
@@ -80,7 +80,7 @@ def build_layer_on_device(G, torch, dev, h, N, sparsity, seed, weight_std=0.02, 
         A.mul_(torch.rand((M, K), generator=gen, device=dev) >= sparsity)
         A = A.to(torch.float16)
         items, offsets = G.encode_on_device(A)
-        mats[name] = (items, offsets, M, K, G.SpMM_SuggestSplitK(M, N, K))
+        mats[name] = (items, offsets, M, K, G.SpMM_SuggestSplitK_Bytes(M, N, K, items.numel() // 4))
         if sample_rows:
             rows = torch.randperm(M, generator=gen, device=dev)[:sample_rows].sort().values
             samples[name] = (rows.cpu().numpy(), A[rows].cpu().numpy())

@@ -22,7 +22,7 @@ Loader = what the patched FasterTransformer does with those files
 the sparse pair of files, whose lengths are the list entries; otherwise the dense file.
 
 Differences from the reference's script, on purpose:
-  * Split_K comes from the library's planner for the 256-CU part (SpMM_SuggestSplitK) instead
+  * Split_K comes from the library's planner for the 256-CU part (SpMM_SuggestSplitK_Bytes) instead
     of the table keyed by M (:20).
   * `orientation="ft"` (default) treats `<name>.bin` as what phase 1 wrote, [K inputs][M
     outputs] (huggingface_opt_convert_Phase1.py:195-271 permutes every weight to that), and
@@ -157,7 +157,8 @@ def convert_model_dir(model_dir, infer_gpu_num, processes=1, tokens=16, orientat
                 M, K = shapes[k]
                 nnz.append(r["nnz"])
                 noff.append(r["num_offsets"])
-                splitk.append(G.SpMM_SuggestSplitK(M, tokens, K) if r["replaced"] else 0)
+                # (the planner is told how much the weight holds: nnz words = nnz / 4 vectors)
+                splitk.append(G.SpMM_SuggestSplitK_Bytes(M, tokens, K, r["nnz"] // 4) if r["replaced"] else 0)
                 (replaced if r["replaced"] else skipped)[k] += 1
         for name, vals in (("NNZ_List", nnz), ("NumOffsets_List", noff), ("SplitK_List", splitk)):
             np.array(vals, dtype=np.int32).tofile(os.path.join(rank_dir, f"{name}.{i}.bin"))
@@ -231,7 +232,7 @@ def upload_layers(layers, device, tokens=None):
         d = {}
         for name, m in zip(("qkv", "out", "ffn1", "ffn2"), mats):
             if m.split_k != 0:
-                s = G.SpMM_SuggestSplitK(m.M, tokens, m.K) if tokens else m.split_k
+                s = G.SpMM_SuggestSplitK_Bytes(m.M, tokens, m.K, len(m.items) // 4) if tokens else m.split_k
                 items = torch.from_numpy(np.array(m.items).view(np.int32)).to(device)
                 if items.numel() == 0:
                     items = torch.zeros(4, dtype=torch.int32, device=device)

@@ -36,6 +36,7 @@ EXPORTED_SYMBOLS = (
     "SpMM_FreeHost",
     "SpMM_GetErrorString",
     "SpMM_SuggestSplitK",
+    "SpMM_SuggestSplitK_Bytes",
     "SpMM_PlanLaunch",
     "SpMM_SplitK_API_Planned",
     "SpMM_SplitK_API_RowMajor",
@@ -120,6 +121,8 @@ def load_library():
     lib.SpMM_GetErrorString.argtypes = [ctypes.c_int]
     lib.SpMM_SuggestSplitK.restype = ctypes.c_int
     lib.SpMM_SuggestSplitK.argtypes = [ctypes.c_int] * 3
+    lib.SpMM_SuggestSplitK_Bytes.restype = ctypes.c_int
+    lib.SpMM_SuggestSplitK_Bytes.argtypes = [ctypes.c_int] * 3 + [ctypes.c_long]
     lib.SpMM_PlanLaunch.restype = ctypes.c_int
     lib.SpMM_PlanLaunch.argtypes = [ctypes.c_int] * 4 + [_i32p] * 4 + [ctypes.POINTER(ctypes.c_double)]
     lib.SpMM_SplitK_API_Planned.restype = ctypes.c_int
@@ -326,6 +329,11 @@ def GenSparseMatrixBinFile(DenseMatrixFileName, M, K, NZWeightsFileName, TileOff
 
 def SpMM_SuggestSplitK(M_Global, N_Global, K_Global):
     return load_library().SpMM_SuggestSplitK(M_Global, N_Global, K_Global)
+
+
+def SpMM_SuggestSplitK_Bytes(M_Global, N_Global, K_Global, Vectors):
+    """SpMM_SuggestSplitK for a weight whose TileOffsets end at `Vectors`."""
+    return load_library().SpMM_SuggestSplitK_Bytes(M_Global, N_Global, K_Global, int(Vectors))
 
 
 def SpMM_PlanLaunch(M_Global, N_Global, K_Global, Split_K):

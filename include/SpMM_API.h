@@ -224,6 +224,18 @@ SPMM_EXPORT const char* SpMM_GetErrorString(int code);
 SPMM_EXPORT int SpMM_SuggestSplitK(int M_Global, int N_Global, int K_Global);
 
 /*
+ * SpMM_SuggestSplitK for a caller that knows how much the weight holds: Vectors = the last entry of
+ * its TileOffsets (16-byte vectors of packed words; a converter has it at hand when it writes
+ * SplitK_List, huggingface_opt_convert_Phase2.py:189-195).  Optima measured at 70, 80 and 90 %
+ * sparsity are built in for the OPT-30B and OPT-66B shapes; the weight's bytes per tile pick the
+ * table (boundaries at 75 and 85 %), other shapes go through the cost model with their real bytes
+ * per tile.  A later SpMM_SplitK_API call with that Split_K finds the matching launch shape again
+ * (it searches every table for the shape and Split_K).  Vectors <= 0 = not known (same as
+ * SpMM_SuggestSplitK).  Returns 1 for shapes the kernels do not take.
+ */
+SPMM_EXPORT int SpMM_SuggestSplitK_Bytes(int M_Global, int N_Global, int K_Global, long Vectors);
+
+/*
  * The launch shape SpMM_SplitK_API uses for (M, N, K, Split_K):
  *   Mode 0  the Waves waves of a workgroup take consecutive 128-row tile rows of one
  *           split-K batch (StageB = 1, up to 16 tokens: they share the batch's activation slice,

@@ -82,7 +82,7 @@ def test_feed_forward_sparsity_sweep(spmm, oracle, M, K, sparsity, skew):
     d_offs = torch.from_numpy(offsets).to(dev)
     rows = np.sort(np.random.default_rng(M + K).choice(M, size=96, replace=False))
     for N in (8, 16, 32, 64):
-        split_k = spmm.SpMM_SuggestSplitK(M, N, K)
+        split_k = spmm.SpMM_SuggestSplitK_Bytes(M, N, K, int(offsets[-1]))
         _sampled_rows_and_linearity(spmm, oracle, torch, A, d_items, d_offs, M, K, N, split_k, rows,
                                     f"feed-forward {sparsity:.0%}{' skewed' if skew else ''}")
 

@@ -68,7 +68,7 @@ def test_converter_writes_the_reference_file_set(tmp_path, spmm, oracle, g):
                 sizes = np.fromfile(stem + ".OutputSizes.bin", dtype=np.int32)
                 assert sizes.tolist() == [o_items.size, o_offs.size] == [nnz, noff]
                 assert nnz == 4 * o_offs[-1] and noff == (M // 128) * (K // 64) + 2
-                assert s == spmm.SpMM_SuggestSplitK(M, 16, K) and s >= 1
+                assert s == spmm.SpMM_SuggestSplitK_Bytes(M, 16, K, nnz // 4) and s >= 1
                 # the dense file is untouched without artificial sparsity
                 assert np.array_equal(np.fromfile(stem + ".bin", dtype=np.float16).view(np.uint16),
                                       weights[(i, j, k)].view(np.uint16).ravel())
