@@ -15,9 +15,9 @@ Prints ONE JSON line:
   value           effective TFLOPS, 2*M*N*K / step time (whole call)
   hbm_gbps        compressed-weight bytes / step time
   roofline        the main kernel alone: algorithmic bytes (16 * TileOffsets[last])
-                  / its average duration, from HIP events recorded on the launch stream
-                  around blocks of K back-to-back launches of it (--repeats blocks enqueued
-                  without a host synchronisation in between; the median block), against the
+                  / its average duration, from two HIP events recorded on the launch stream
+                  around --repeats x K back-to-back launches of it (one pair of events: an
+                  event between two kernels costs the stream microseconds), against the
                   8 TB/s HBM peak
   cpu_baseline    the CPU path timed on this host: reference encoder (oracle/_ref,
                   single thread) + fp32-accumulate dense GEMM (oracle, single thread)
@@ -146,24 +146,6 @@ def events_ms(lib, sptr, call, n):
     ms = float(lib.SpMM_EventElapsedMs(ev0, ev1))
     lib.SpMM_EventDestroy(ev0)
     lib.SpMM_EventDestroy(ev1)
-    return ms
-
-
-def chained_events_ms(lib, sptr, call, n, blocks):
-    """`blocks` blocks of n calls enqueued back to back, an event between every two blocks and
-    no host synchronisation in between: the milliseconds of each block, with the stream kept busy
-    throughout (so no block pays the start-up latency of a launch into an idle queue)."""
-    events = [lib.SpMM_EventCreate() for _ in range(blocks + 1)]
-    lib.SpMM_EventRecord(events[0], sptr)
-    k = 0
-    for b in range(blocks):
-        for _ in range(n):
-            call(k)
-            k += 1
-        lib.SpMM_EventRecord(events[b + 1], sptr)
-    ms = [float(lib.SpMM_EventElapsedMs(events[b], events[b + 1])) for b in range(blocks)]
-    for e in events:
-        lib.SpMM_EventDestroy(e)
     return ms
 
 
@@ -298,6 +280,8 @@ def main():
     ap.add_argument("--no-reorder", action="store_true",
                     help="encode with InitSparseMatrixA_API_NoReorder (the reference's ablation of its bank-aware reordering)")
     ap.add_argument("--repeats", type=int, default=15, help="timed blocks of --steps steps; the median is reported")
+    ap.add_argument("--prewarm-seconds", type=float, default=PREWARM_SECONDS,
+                    help="untimed launches before --warmup, to settle the clocks (shorten it under a counter-collecting profiler)")
     ap.add_argument("--no-sweep", action="store_true", help="skip the other configurations after the headline")
     ap.add_argument("--no-stack", action="store_true", help="sweep without the 64-layer decoder stack (52 GB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -385,7 +369,24 @@ def main():
             sys.exit(1)
 
     # ---- settle the clocks: the same call, untimed, for a fixed wall time whatever --warmup says
-    prewarm_launches = prewarm(step, torch)
+    # (after an idle spell this GPU needs some 10 ms of continuous launches to reach its clocks)
+    prewarm_launches = prewarm(step, torch, args.prewarm_seconds)
+
+    # ---- the main kernel alone, live: back-to-back launches of it (no reduction in between)
+    # bracketed by two HIP events recorded on the launch stream, straight after the pre-warm; the
+    # average includes the dispatch gap between consecutive kernels but no per-launch event
+    # overhead.  --repeats x K launches between ONE pair of events: recording an event between two
+    # kernels costs the stream a few microseconds, which at K = 20 would add 1-2 % to every block
+    # timed on its own.
+    def partials(i):
+        rc = lib.SpMM_SplitK_Partials(sptr, p_items[i % copies], p_offs[i % copies], p_B, p_W, M, N, K, split_k)
+        if rc:
+            raise RuntimeError(f"SpMM_SplitK_Partials -> {rc}")
+
+    for i in range(200):
+        partials(i)
+    kernel_launches = args.steps * max(1, args.repeats)
+    kernel_ms_avg = events_ms(lib, sptr, partials, kernel_launches) / kernel_launches
 
     # ---- timed region: W warm-up steps, then exactly K steps between synchronisations; that
     # block is timed --repeats times (each with its own synchronisations) and the median reported
@@ -401,20 +402,6 @@ def main():
         torch.cuda.synchronize()
         blocks_ms.append((time.perf_counter() - t0) * 1e3)
     ms_per_step = float(np.median(blocks_ms)) / args.steps
-
-    # ---- the main kernel alone, live: K back-to-back launches of it (no reduction in between)
-    # bracketed by two HIP events recorded on the launch stream; the average includes the
-    # dispatch gap between consecutive kernels but no per-launch event overhead.
-    def partials(i):
-        rc = lib.SpMM_SplitK_Partials(sptr, p_items[i % copies], p_offs[i % copies], p_B, p_W, M, N, K, split_k)
-        if rc:
-            raise RuntimeError(f"SpMM_SplitK_Partials -> {rc}")
-
-    for i in range(200):
-        partials(i)
-    kernel_blocks_ms = chained_events_ms(lib, sptr, partials, args.steps, max(1, args.repeats))
-    kernel_ms_avg = float(np.median(kernel_blocks_ms)) / args.steps
-    torch.cuda.synchronize()
 
     for i in range(args.calibration_copies):
         src, dst = d_items[i % copies], d_items[(i + 1) % copies]  # all copies hold the same bytes
@@ -439,7 +426,7 @@ def main():
         "ms_per_step": ms_per_step,
         "timing": {"repeats": len(blocks_ms), "statistic": "median of the timed blocks of --steps steps",
                    "block_ms_min": float(min(blocks_ms)), "block_ms_max": float(max(blocks_ms)),
-                   "prewarm_launches": prewarm_launches, "prewarm_seconds": PREWARM_SECONDS},
+                   "prewarm_launches": prewarm_launches, "prewarm_seconds": args.prewarm_seconds},
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -470,6 +457,7 @@ def main():
             "traffic_source": TRAFFIC_SOURCE,
             "kernel": "tcsl_spmm_kernel",
             "kernel_ms_avg": kernel_ms_avg,
+            "kernel_launches_timed": kernel_launches,
             "algorithmic_bytes_per_launch": a_bytes,
         },
         "check": check,
