@@ -22,6 +22,21 @@
 //   two positions of a group are different and ascending.  A group with fewer than two kept values
 //   is filled with zero values at free positions.
 //   1.125 bytes per dense element whatever the sparsity.
+//
+// The residual (what a group of four holds beyond its first two kept values) for the launch that
+// multiplies both parts at once: one list of 32-bit words per record, numbered like the records
+// (record_index), lists stored one after the other in that order, so that the lists of a group of
+// eight row blocks for one unit are neighbours, like their records.
+//   word    = fp16 value | address << 16
+//   address = byte address of element (row r, column c) of the record's 16 x 128 block in the dense
+//             image the kernel keeps in LDS: r * 256 + (((c / 8) ^ r) << 4) + (c % 8) * 2  (the 16-byte
+//             granules of a row are permuted by the row number, so that the sixteen rows' granules
+//             of one column group fall into sixteen different bank groups)
+//   Offsets[i] .. Offsets[i + 1] are list i's words (records + 1 entries, 32-bit).  The words of a
+//   list are read 64 at a time, one per lane; they are ordered so that each such round spreads
+//   over the LDS banks (words that share a bank are dealt to different rounds).  The array of
+//   words is followed by 64 words of padding.
+// 4 bytes per kept residual value.
 #pragma once
 #include <cstdint>
 
@@ -46,6 +61,15 @@ int pack(const uint16_t* A1, int M, int K, uint8_t* packed);
 inline long record_index(long row_block, int unit, int units)
 {
     return ((row_block / kGroupBlocks) * units + unit) * kGroupBlocks + row_block % kGroupBlocks;
+}
+// Residual lists of a row-major M x K matrix (the A2 of decompose; any matrix with at most 1024
+// kept values per 16 x 128 block works).  *words and *offsets are malloc'ed (caller frees);
+// *longest = the longest list's length.  Returns the number of offsets or a negative code.
+int pack_residual(const uint16_t* A2, int M, int K, uint32_t** words, int** offsets, int* longest);
+constexpr int kListPadWords = 64;
+inline uint32_t residual_address(int row, int col)
+{
+    return static_cast<uint32_t>(row * 256 + ((((col >> 3) ^ row) & 15) << 4) + (col & 7) * 2);
 }
 inline long bytes(int M, int K)
 {

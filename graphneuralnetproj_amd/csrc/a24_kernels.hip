@@ -234,15 +234,28 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_kernel(const uint8_t* __res
 // from LDS instead of the L2, and no sum across waves is needed at the end.
 constexpr int kRowBytes = 272;
 
-template<int NT, int RB, int W>
+// With RL > 0 the same launch also multiplies the residual (what the split leaves beyond two kept
+// values per group of four), so that C = A1*B + A2*B costs one pass over the activations instead of
+// two kernels and a sum.  The residual comes as one list of words per record (a24_format.h:
+// fp16 value | byte address in a 16 x 128 image << 16), at most RL * 64 words each.  A wave
+// scatters a list into its own 4 KiB LDS image (ds_write_b16; lanes past the end repeat the last
+// word), reads the image back as dense MFMA operands, writes zeros where it wrote values, and runs
+// v_mfma_f32_16x16x32_f16 on the same activation fragments and accumulators as the sparse
+// instruction.  The lists' offsets travel one unit ahead of the words, on the vector path like
+// everything else, so that every unit issues the same number of loads.
+constexpr int kImageBytes = 4096;
+
+template<int NT, int RB, int W, int RL>
 __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8_t* __restrict__ packed,
                                                                      const _Float16* __restrict__ B,
                                                                      _Float16* __restrict__ out, int units,
                                                                      int units_per_batch, long ldb, long ldo, long slab,
-                                                                     int n_tokens)
+                                                                     int n_tokens, const unsigned* __restrict__ words,
+                                                                     const int* __restrict__ offsets)
 {
-    extern __shared__ __attribute__((aligned(16))) unsigned char tile[];  // [2][NT * 16][kRowBytes]
+    extern __shared__ __attribute__((aligned(16))) unsigned char tile[];  // [2][NT * 16][kRowBytes], then [W][kImageBytes]
     constexpr int kBuf = NT * 16 * kRowBytes;
+    constexpr int RLA = RL > 0 ? RL : 1;
     constexpr int kThreads = W * kWave;
     constexpr int CH = (NT * 256 + kThreads - 1) / kThreads;  // 16-byte chunks of a tile per thread
     const int tid = threadIdx.x;
@@ -276,12 +289,19 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
         frag[t] = n * kRowBytes + (lane >> 4) * 16;
     }
 
-    float4v acc[RB][NT];
+    // The residual's dense products get accumulators of their own, added to the others at the end:
+    // a dense MFMA that takes the sparse instruction's result as its addend directly behind it read
+    // the last two of the four registers before they were written (the compiler places no wait
+    // between the two kinds; chains of one kind are fine).
+    float4v acc[RB][NT], accd[RL > 0 ? RB : 1][NT];
 #pragma unroll
     for (int r = 0; r < RB; r++)
 #pragma unroll
-        for (int t = 0; t < NT; t++)
+        for (int t = 0; t < NT; t++) {
             acc[r][t] = float4v{0.f, 0.f, 0.f, 0.f};
+            if constexpr (RL > 0)
+                accd[r][t] = float4v{0.f, 0.f, 0.f, 0.f};
+        }
 
     // Three rotating sets of "unit registers": the records of RB row blocks and this thread's chunks
     // of the activation tile.  (A thread beyond the tile's last chunk repeats one of token 0's: the
@@ -289,15 +309,49 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
     struct UnitRegs {
         AFrag a[RB];
         u32x4 stage[CH];
+        unsigned w[RB][RLA];  // residual words of the unit's RB lists
+        int next;             // lane j <= RB: offsets[first record of the unit after this one + j]
+        int count[RB];        // words in each list (the same in every lane)
     };
-    constexpr int kLoadsA = 3 * RB;      // loads of one unit's records per lane
-    auto issue_unit = [&](UnitRegs& x, int unit) {  // activation chunks first: they are needed first
+    constexpr int kLoadsA = (3 + RL) * RB;      // loads of one unit's records and lists per lane
+    constexpr int kLoadsHead = RL > 0 ? 1 : 0;  // the offsets load that leads a unit's loads
+    // lists are numbered like records: this wave's RB lists of a unit are neighbours
+    const long list0 = ((long)(block0 / kGroupBlocks) * units) * kGroupBlocks + block0 % kGroupBlocks;
+    const int* const off_lane = offsets + list0 + (lane <= RB ? lane : RB);
+    unsigned char* const image = tile + 2 * kBuf + wave * kImageBytes;
+    // o[0..RB]: the offsets of `unit`'s lists, the same in every lane
+    auto issue_unit = [&](UnitRegs& x, int unit, int unit_after, const int (&o)[RB + 1]) {
+        if constexpr (RL > 0)
+            asm volatile("global_load_dword %0, %1, off" : "=v"(x.next) : "v"(off_lane + (size_t)unit_after * kGroupBlocks));
 #pragma unroll
-        for (int i = 0; i < CH; i++)
+        for (int i = 0; i < CH; i++)  // activation chunks before the records: they are needed first
             x.stage[i] = issue_b(src[i] + (size_t)unit * 128);
 #pragma unroll
         for (int r = 0; r < RB; r++)
             x.a[r] = issue_a(rec[r] + (size_t)unit * kUnitStride + lane * 16, rec[r] + (size_t)unit * kUnitStride + lane * 4);
+        if constexpr (RL > 0) {
+#pragma unroll
+            for (int r = 0; r < RB; r++) {
+                const int n = o[r + 1] - o[r];
+                x.count[r] = n;
+                const int last = n > 0 ? n - 1 : 0;
+#pragma unroll
+                for (int i = 0; i < RL; i++) {
+                    const int at = lane + i * kWave;
+                    const unsigned* p = words + o[r] + (at < last ? at : last);
+                    asm volatile("global_load_dword %0, %1, off nt" : "=v"(x.w[r][i]) : "v"(p));
+                }
+            }
+        }
+    };
+    // The offsets that a unit's `next` load brought, once it has landed.
+    auto offsets_from = [&](UnitRegs& x, int (&o)[RB + 1]) {
+        if constexpr (RL > 0) {
+            settle(x.next);
+#pragma unroll
+            for (int j = 0; j <= RB; j++)
+                o[j] = __builtin_amdgcn_readlane(x.next, j);
+        }
     };
     auto store_b = [&](UnitRegs& x, int buf) {
 #pragma unroll
@@ -312,9 +366,39 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
             settle(x.a[r].v[0]);
             settle(x.a[r].v[1]);
             settle(x.a[r].idx);
+            if constexpr (RL > 0) {
+#pragma unroll
+                for (int i = 0; i < RL; i++)
+                    settle(x.w[r][i]);
+            }
         }
     };
-    auto multiply_from = [&](const AFrag(&a)[RB], int buf) {
+    // where this lane's dense operands sit in the image: row lane % 16, granule (4 s + lane / 16) ^ row
+    const int img_row = (lane & 15) * 256;
+    auto multiply_from = [&](UnitRegs& x, int buf) {
+        const AFrag(&a)[RB] = x.a;
+        half8 dense[RB][4];
+        if constexpr (RL > 0) {
+            // One list after the other through the wave's image: LDS operations of a wave run in
+            // order, so values, read-back and zeros need no barrier.
+#pragma unroll
+            for (int r = 0; r < RB; r++) {
+                const int n = x.count[r];
+                if (n > 0) {
+#pragma unroll
+                    for (int i = 0; i < RL; i++)
+                        if (i == 0 || n > i * kWave)
+                            *reinterpret_cast<unsigned short*>(image + (x.w[r][i] >> 16)) = static_cast<unsigned short>(x.w[r][i]);
+#pragma unroll
+                    for (int s = 0; s < 4; s++)
+                        dense[r][s] = *reinterpret_cast<const half8*>(image + img_row + (((s * 4 + (lane >> 4)) ^ (lane & 15)) << 4));
+#pragma unroll
+                    for (int i = 0; i < RL; i++)
+                        if (i == 0 || n > i * kWave)
+                            *reinterpret_cast<unsigned short*>(image + (x.w[r][i] >> 16)) = 0;
+                }
+            }
+        }
 #pragma unroll
         for (int t = 0; t < NT; t++) {
             half8 f[4];
@@ -327,6 +411,13 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
                 acc[r][t] = __builtin_amdgcn_smfmac_f32_16x16x32_f16(step_values(a[r], 1), f[1], acc[r][t], (int)a[r].idx, 0, 1);
                 acc[r][t] = __builtin_amdgcn_smfmac_f32_16x16x32_f16(step_values(a[r], 2), f[2], acc[r][t], (int)a[r].idx, 0, 2);
                 acc[r][t] = __builtin_amdgcn_smfmac_f32_16x16x32_f16(step_values(a[r], 3), f[3], acc[r][t], (int)a[r].idx, 0, 3);
+                if constexpr (RL > 0) {
+                    if (x.count[r] > 0) {
+#pragma unroll
+                        for (int s = 0; s < 4; s++)
+                            accd[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dense[r][s], f[s], accd[r][t], 0, 0, 0);
+                    }
+                }
             }
         }
     };
@@ -342,9 +433,30 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
     if (u < u1) {
         const int last = u1 - 1;
         auto ahead = [&](int d) { return u + d < last ? u + d : last; };
-        issue_unit(x[0], u);
-        issue_unit(x[1], ahead(1));
-        wait_loads<kLoadsA + CH + kLoadsA>();  // the first tile
+        int o[RB + 1] = {};
+        if constexpr (RL > 0) {
+            // the image starts out clear; the first two units' offsets are fetched by themselves
+            for (int i = lane * 16; i < kImageBytes; i += kWave * 16)
+                *reinterpret_cast<u32x4*>(image + i) = u32x4{0u, 0u, 0u, 0u};
+            int first, second;
+            asm volatile("global_load_dword %0, %1, off" : "=v"(first) : "v"(off_lane + (size_t)u * kGroupBlocks));
+            asm volatile("global_load_dword %0, %1, off" : "=v"(second) : "v"(off_lane + (size_t)ahead(1) * kGroupBlocks));
+            wait_loads<0>();
+            settle(first);
+            settle(second);
+#pragma unroll
+            for (int j = 0; j <= RB; j++)
+                o[j] = __builtin_amdgcn_readlane(first, j);
+            issue_unit(x[0], u, ahead(1), o);
+#pragma unroll
+            for (int j = 0; j <= RB; j++)
+                o[j] = __builtin_amdgcn_readlane(second, j);
+            issue_unit(x[1], ahead(1), ahead(2), o);
+        } else {
+            issue_unit(x[0], u, u, o);
+            issue_unit(x[1], ahead(1), u, o);
+        }
+        wait_loads<kLoadsA + kLoadsHead + CH + kLoadsA>();  // the first tile
         store_b(x[0], 0);
         __syncthreads();
         auto phase = [&](auto kc) {  // unit u, whose registers are set kc
@@ -353,8 +465,10 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
             wait_loads<kLoadsA>();
             landed(x[k]);
             store_b(x[(k + 1) % 3], buf ^ 1);
-            issue_unit(x[(k + 2) % 3], ahead(2));
-            multiply_from(x[k].a, buf);
+            int o2[RB + 1] = {};
+            offsets_from(x[(k + 1) % 3], o2);  // unit u + 1 brought the offsets of unit u + 2
+            issue_unit(x[(k + 2) % 3], ahead(2), ahead(3), o2);
+            multiply_from(x[k], buf);
             __syncthreads();
             ++u;
         };
@@ -381,6 +495,8 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
 #pragma unroll
             for (int i = 0; i < CH; i++)
                 settle(x[k].stage[i]);
+            if constexpr (RL > 0)
+                settle(x[k].next);
         }
     }
 
@@ -391,7 +507,9 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
         for (int t = 0; t < NT; t++) {
             const int n = t * 16 + (lane & 15);
             if (n < n_tokens) {
-                const float4v s = acc[r][t];
+                float4v s = acc[r][t];
+                if constexpr (RL > 0)
+                    s += accd[r][t];
                 half4 h = {static_cast<_Float16>(s[0]), static_cast<_Float16>(s[1]), static_cast<_Float16>(s[2]),
                            static_cast<_Float16>(s[3])};
                 *reinterpret_cast<half4*>(dstc + (size_t)n * ldo + (block0 + r) * 16 + (lane >> 4) * 4) = h;
@@ -400,30 +518,42 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
     }
 }
 
-template<int NT, int RB, int W>
+template<int NT, int RB, int W, int RL>
 int launch_shared_b(hipStream_t stream, const void* packed, const void* B, void* out, int M, int N, int K, int split_k,
-                    long ldb, long ldo, long slab)
+                    long ldb, long ldo, long slab, const void* words, const void* offsets)
 {
     const int units = K / 128;
     const int per_batch = (units + split_k - 1) / split_k;
     if (M % (16 * RB * W) != 0)
         return static_cast<int>(hipErrorInvalidValue);
-    hipLaunchKernelGGL((a24_spmm_shared_b_kernel<NT, RB, W>), dim3(M / (16 * RB * W), split_k), dim3(W * kWave),
-                       2 * NT * 16 * kRowBytes, stream, static_cast<const uint8_t*>(packed), static_cast<const _Float16*>(B),
-                       static_cast<_Float16*>(out), units, per_batch, ldb, ldo, slab, N);
+    const unsigned lds = 2 * NT * 16 * kRowBytes + (RL > 0 ? W * kImageBytes : 0);
+    auto kern = a24_spmm_shared_b_kernel<NT, RB, W, RL>;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess)
+            return static_cast<int>(e);
+    }
+    hipLaunchKernelGGL(kern, dim3(M / (16 * RB * W), split_k), dim3(W * kWave), lds, stream,
+                       static_cast<const uint8_t*>(packed), static_cast<const _Float16*>(B), static_cast<_Float16*>(out), units,
+                       per_batch, ldb, ldo, slab, N, static_cast<const unsigned*>(words), static_cast<const int*>(offsets));
     return static_cast<int>(hipGetLastError());
 }
 
+// rl: loads per residual list (0 = no residual).  The fused form has the library's own launch
+// shapes only: two row blocks per wave, four or eight waves.
 template<int NT>
 int launch_shared_b_nt(hipStream_t s, const void* packed, const void* B, void* out, int M, int N, int K, int split_k, int rb,
-                       int waves, long ldb, long ldo, long slab)
+                       int waves, long ldb, long ldo, long slab, int rl, const void* words, const void* offsets)
 {
-#define A24_CASE(RB_, W_)         \
-    if (rb == RB_ && waves == W_) \
-        return launch_shared_b<NT, RB_, W_>(s, packed, B, out, M, N, K, split_k, ldb, ldo, slab);
-    A24_CASE(2, 4) A24_CASE(2, 8)
-    if constexpr (NT <= 2) {  // three record sets of four row blocks do not fit the registers beside 64 tokens
-        A24_CASE(4, 2) A24_CASE(4, 4) A24_CASE(4, 8)
+#define A24_CASE(RB_, W_, RL_)                   \
+    if (rb == RB_ && waves == W_ && rl == RL_) \
+        return launch_shared_b<NT, RB_, W_, RL_>(s, packed, B, out, M, N, K, split_k, ldb, ldo, slab, words, offsets);
+    A24_CASE(2, 4, 0) A24_CASE(2, 8, 0)
+    A24_CASE(2, 4, 1) A24_CASE(2, 8, 1) A24_CASE(2, 4, 2) A24_CASE(2, 8, 2) A24_CASE(2, 4, 3) A24_CASE(2, 8, 3)
+    A24_CASE(2, 4, 4)
+    if constexpr (NT <= 2) {
+        A24_CASE(2, 8, 4)  // with 64 tokens it would not fit 256 registers  // three record sets of four row blocks do not fit the registers beside 64 tokens
+        A24_CASE(4, 2, 0) A24_CASE(4, 4, 0) A24_CASE(4, 8, 0)
     }
 #undef A24_CASE
     return static_cast<int>(hipErrorInvalidValue);
@@ -467,19 +597,24 @@ int launch_nt(hipStream_t s, const void* packed, const void* B, void* out, int M
 
 // Batch b of ceil((K/128)/split_k) units writes fp16 [N][ldo] to out + b * slab.  The caller has
 // checked: M % (16 * rb) == 0 (share_b: M % (16 * rb * waves) == 0), K % 128 == 0, N in {8, 16, 32, 64}, no batch empty, pointers set.
+// residual_loads > 0 (share_b with rb == 2 only): the launch also multiplies the residual lists
+// words / offsets, none longer than 64 * residual_loads words.
 extern "C" int a24_launch_spmm(void* stream, const void* packed, const void* B, void* out, int M, int N, int K,
-                               int split_k, int rb, int waves, int share_b, long ldb, long ldo, long slab)
+                               int split_k, int rb, int waves, int share_b, long ldb, long ldo, long slab,
+                               int residual_loads, const void* words, const void* offsets)
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (share_b) {  // waves own rows and share the activation tile through LDS
         switch (N) {
             case 8:
-            case 16: return launch_shared_b_nt<1>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab);
-            case 32: return launch_shared_b_nt<2>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab);
-            case 64: return launch_shared_b_nt<4>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab);
+            case 16: return launch_shared_b_nt<1>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets);
+            case 32: return launch_shared_b_nt<2>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets);
+            case 64: return launch_shared_b_nt<4>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets);
             default: return static_cast<int>(hipErrorInvalidValue);
         }
     }
+    if (residual_loads != 0)
+        return static_cast<int>(hipErrorInvalidValue);
     switch (N) {
         case 8:
         case 16: return launch_nt<1>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab);

@@ -1,6 +1,8 @@
 // Host side of the 2:4 + residual path: the reference's split of a weight into a part for
 // sparse matrix cores and a Tiled-CSL residual, and the packer of the first part's records.
+#include <algorithm>
 #include <atomic>
+#include <cstdlib>
 #include <cstring>
 #include <thread>
 #include <vector>
@@ -126,6 +128,125 @@ int pack(const uint16_t* A1, int M, int K, uint8_t* packed)
         }
     });
     return bad.load() ? kErrNotTwoOfFour : 0;
+}
+
+namespace {
+
+// Orders one list's words so that every round of 64 (one word per lane; the last round may be
+// partial) spreads over the 64 LDS banks: banks are taken fullest first, and each of a bank's
+// words goes to the round that holds the fewest words of that bank so far and still has room
+// (the emptier round on a tie).
+void order_by_bank(std::vector<uint32_t>& list, std::vector<uint32_t>& tmp)
+{
+    const int n = static_cast<int>(list.size());
+    const int rounds = (n + 63) / 64;
+    if (rounds <= 1)
+        return;
+    auto bank_of = [](uint32_t w) { return static_cast<int>(((w >> 16) >> 2) & 63); };
+    int count[64] = {};
+    for (uint32_t w : list)
+        count[bank_of(w)]++;
+    int order[64];
+    for (int b = 0; b < 64; b++)
+        order[b] = b;
+    std::stable_sort(order, order + 64, [&](int a, int b) { return count[a] > count[b]; });
+    int start[64], at = 0;  // where each bank's words begin in the bank-sorted sequence
+    for (int i = 0; i < 64; i++) {
+        start[order[i]] = at;
+        at += count[order[i]];
+    }
+    tmp.assign(n, 0);
+    int fill[64];
+    for (int b = 0; b < 64; b++)
+        fill[b] = start[b];
+    for (uint32_t w : list)
+        tmp[fill[bank_of(w)]++] = w;
+    std::vector<int> used(rounds, 0), mine(rounds);
+    for (int i = 0; i < 64; i++) {
+        const int b = order[i];
+        std::fill(mine.begin(), mine.end(), 0);
+        for (int j = 0; j < count[b]; j++) {
+            int best = -1, best_free = 0;
+            for (int r = 0; r < rounds; r++) {
+                const int free = (r == rounds - 1 ? n - 64 * (rounds - 1) : 64) - used[r];
+                if (free > 0 && (best < 0 || mine[r] < mine[best] || (mine[r] == mine[best] && free > best_free))) {
+                    best = r;
+                    best_free = free;
+                }
+            }
+            list[best * 64 + used[best]++] = tmp[start[b] + j];
+            mine[best]++;
+        }
+    }
+}
+
+}  // namespace
+
+int pack_residual(const uint16_t* A2, int M, int K, uint32_t** words, int** offsets, int* longest)
+{
+    if (!A2 || !words || !offsets || !longest)
+        return kErrNullPointer;
+    if (M <= 0 || K <= 0 || M % (kRows * kGroupBlocks) != 0 || K % kUnitCols != 0)
+        return kErrBadShape;
+    const int units = K / kUnitCols;
+    const long blocks = M / kRows;
+    const long records = blocks * units;
+    if (records + 1 > 0x7fffffffL)
+        return kErrBadShape;
+    int* off = static_cast<int*>(std::malloc((records + 1) * sizeof(int)));
+    if (!off)
+        return kErrNoMemory;
+    // pass 1: list lengths, by list number
+    parallel_for(blocks, [=](long b0, long b1) {
+        for (long rb = b0; rb < b1; rb++)
+            for (int u = 0; u < units; u++) {
+                int n = 0;
+                for (int r = 0; r < kRows; r++) {
+                    const uint16_t* row = A2 + (rb * kRows + r) * static_cast<long>(K) + static_cast<long>(u) * kUnitCols;
+                    for (int c = 0; c < kUnitCols; c++)
+                        n += kept(row[c]) ? 1 : 0;
+                }
+                off[record_index(rb, u, units) + 1] = n;
+            }
+    });
+    off[0] = 0;
+    int most = 0;
+    long total = 0;
+    for (long i = 1; i <= records; i++) {
+        most = off[i] > most ? off[i] : most;
+        total += off[i];
+        if (total > 0x7fffffffL - kListPadWords) {
+            std::free(off);
+            return kErrBadShape;
+        }
+        off[i] = static_cast<int>(total);
+    }
+    uint32_t* out = static_cast<uint32_t*>(std::malloc((total + kListPadWords) * sizeof(uint32_t)));
+    if (!out) {
+        std::free(off);
+        return kErrNoMemory;
+    }
+    std::memset(out + total, 0, kListPadWords * sizeof(uint32_t));
+    // pass 2: the words
+    parallel_for(blocks, [=](long b0, long b1) {
+        std::vector<uint32_t> list, tmp;
+        for (long rb = b0; rb < b1; rb++)
+            for (int u = 0; u < units; u++) {
+                list.clear();
+                for (int r = 0; r < kRows; r++) {
+                    const uint16_t* row = A2 + (rb * kRows + r) * static_cast<long>(K) + static_cast<long>(u) * kUnitCols;
+                    for (int c = 0; c < kUnitCols; c++)
+                        if (kept(row[c]))
+                            list.push_back(row[c] | residual_address(r, c) << 16);
+                }
+                order_by_bank(list, tmp);
+                std::memcpy(out + off[record_index(rb, u, units)], list.data(), list.size() * sizeof(uint32_t));
+            }
+    });
+    *words = out;
+    *offsets = off;
+    *longest = most;
+    return static_cast<int>(records + 1);
 }
 
 }  // namespace a24

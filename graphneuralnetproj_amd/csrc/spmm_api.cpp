@@ -22,7 +22,8 @@ int tcsl_launch_copy(void* stream, void* dst, const void* src, long bytes);
 int tcsl_launch_encode_offsets(void* stream, const void* A, int M, int K, int* offsets);
 int tcsl_launch_encode_items(void* stream, const void* A, int M, int K, const int* offsets, void* items);
 int a24_launch_spmm(void* stream, const void* packed, const void* B, void* out, int M, int N, int K, int split_k, int rb,
-                    int waves, int share_b, long ldb, long ldo, long slab);
+                    int waves, int share_b, long ldb, long ldo, long slab, int residual_loads = 0,
+                    const void* words = nullptr, const void* offsets = nullptr);
 int a24_launch_split_pack(void* stream, const void* A, void* packed, void* residual, int M, int K);
 int a24_side_begin(void* stream, void** side);
 int a24_side_end(void* stream, void* side);
@@ -506,7 +507,22 @@ A24Plan a24_default_plan(int M, int N, int K)
             p.split_k = s;
         }
     }
+    // Half the slabs from half as many waves per workgroup: the same number of workgroups, two of
+    // them on a compute unit, and with an even split of two no reduction kernel at all (FFN1
+    // 28672x7168, N = 16: 36.0 us against 35.2 + 3 us).  With 64 tokens eight waves hide the matrix
+    // cores' and the LDS's latencies better (41 us against 46).
+    if (N <= 32 && p.waves == 8 && p.split_k % 2 == 0) {
+        p.waves = 4;
+        p.split_k /= 2;
+    }
     return p;
+}
+
+// Waves per workgroup for a caller-chosen split: eight (256 rows) where that many workgroups still
+// fill the chip, else four.
+int a24_waves_for(int M, int split_k)
+{
+    return (M % 256 == 0 && static_cast<long>(M / 256) * split_k > 160) ? 8 : 4;
 }
 
 bool a24_shape_ok(int M, int N, int K, int split_k, int row_blocks, int waves, int share_b = 0)
@@ -542,7 +558,7 @@ extern "C" int HeteroSparse_A1_Partials(void* stream, const void* Packed_A1, con
     if (RowBlocks == 0 || Waves == 0) {
         const A24Plan d = a24_default_plan(M > 0 ? M : 128, N, K > 0 ? K : 128);
         p.row_blocks = d.row_blocks;
-        p.waves = d.waves;
+        p.waves = a24_waves_for(M > 0 ? M : 128, Split_K);
         p.share_b = d.share_b;
     }
     if (!Packed_A1 || !B || !Partials || !a24_shape_ok(M, N, K, p.split_k, p.row_blocks, p.waves, p.share_b)) {
@@ -570,7 +586,9 @@ extern "C" int HeteroSparse_SpMM_API(void* stream, const void* Packed_A1, const 
         std::printf("MM_Sparse_API Error: Unsupported N dimension %d!\n", N);  // csrc/SpMM_API.cu:192-193
         return tcsl_error_unknown();
     }
-    const A24Plan d = a24_shape_ok(M, N, K, Split_K_A1, 1, 1) ? a24_default_plan(M, N, K) : A24Plan{1, 1, 1};
+    A24Plan d = a24_shape_ok(M, N, K, Split_K_A1, 1, 1) ? a24_default_plan(M, N, K) : A24Plan{1, 1, 1};
+    if (d.share_b)
+        d.waves = a24_waves_for(M, Split_K_A1);
     if (!Packed_A1 || !B || !C || (residual && !TileOffsets_A2) || !a24_shape_ok(M, N, K, Split_K_A1, d.row_blocks, d.waves, d.share_b)
         || (residual && (Split_K_A2 < 1 || Split_K_A2 > 65535)) || ((residual || Split_K_A1 > 1) && !Reduction_Workspace)
         || (Flags & ~HETERO_FLAG_TWO_STREAMS)) {
@@ -625,4 +643,36 @@ extern "C" int HeteroSparse_SpMM_API(void* stream, const void* Packed_A1, const 
     if (fused)
         return 0;
     return tcsl_launch_reduce(stream, C, ws, mn, 1, mn, Split_K_A1 + Split_K_A2, 0);
+}
+
+extern "C" int HeteroSparse_PackA2(const uint16_t* A2_h, int M, int K, uint32_t** Words, int** Offsets, int* LongestList)
+{
+    return a24::pack_residual(A2_h, M, K, Words, Offsets, LongestList);
+}
+
+extern "C" int HeteroSparse_Fused_SpMM_API(void* stream, const void* Packed_A1, const void* A2_Words, const int* A2_Offsets,
+                                           int LongestList, const void* B, void* C, int M, int N, int K,
+                                           void* Reduction_Workspace, int Split_K)
+{
+    if (N != 8 && N != 16 && N != 32 && N != 64) {
+        std::printf("MM_Sparse_API Error: Unsupported N dimension %d!\n", N);  // csrc/SpMM_API.cu:192-193
+        return tcsl_error_unknown();
+    }
+    const A24Plan d = a24_shape_ok(M, N, K, Split_K, 1, 1) ? a24_default_plan(M, N, K) : A24Plan{1, 1, 1};
+    if (!Packed_A1 || !A2_Words || !A2_Offsets || !B || !C || LongestList < 0 || LongestList > HETERO_FUSED_MAX_LIST
+        || !a24_shape_ok(M, N, K, Split_K, d.row_blocks, d.waves, d.share_b) || d.row_blocks != 2 || !d.share_b
+        || (Split_K > 1 && !Reduction_Workspace)) {
+        std::fprintf(stderr, "HeteroSparse_Fused_SpMM_API: unsupported call M=%d N=%d K=%d Split_K=%d LongestList=%d (need M %% 128 == 0, K %% 128 == 0, no empty batch, lists of at most %d words, non-null pointers)\n",
+                     M, N, K, Split_K, LongestList, HETERO_FUSED_MAX_LIST);
+        return tcsl_error_invalid_value();
+    }
+    const int loads = (LongestList + 63) / 64;
+    const long mn = static_cast<long>(M) * N;
+    void* out = Split_K == 1 ? C : Reduction_Workspace;
+    const int waves = (N == 64 && loads == 4) ? 4 : a24_waves_for(M, Split_K);  // the former: what fits the registers
+    const int rc = a24_launch_spmm(stream, Packed_A1, B, out, M, N, K, Split_K, d.row_blocks, waves, d.share_b, K, M, mn,
+                                   loads, A2_Words, A2_Offsets);
+    if (rc != 0 || Split_K == 1)
+        return rc;
+    return tcsl_launch_reduce(stream, C, static_cast<uint16_t*>(Reduction_Workspace), mn, 1, mn, Split_K, 0);
 }

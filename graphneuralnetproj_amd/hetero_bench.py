@@ -10,7 +10,8 @@ weights rotated over several copies so that no cache level holds the stream):
   a1      the 2:4 kernel alone (its bytes do not depend on the sparsity);
   hybrid  HeteroSparse_SpMM_API: 2:4 kernel, then the residual's Tiled-CSL kernel (--residual-split-k), which
           adds all slabs up itself where its launch allows, else one reduction kernel;
-  2-str   the same with HETERO_FLAG_TWO_STREAMS (the two kernels side by side).
+  2-str   the same with HETERO_FLAG_TWO_STREAMS (the two kernels side by side);
+  fused   HeteroSparse_Fused_SpMM_API: both parts in the 2:4 kernel's launch (residual as lists).
 """
 import argparse
 
@@ -60,12 +61,14 @@ def main():
         packed = G.HeteroSparse_PackA1(A1)
         items, offs = G.InitSparseMatrixA_API(A)
         items2, offs2 = G.InitSparseMatrixA_API(A2)
+        words, woffs, longest = G.HeteroSparse_PackA2(A2)
         share = float((A2 != 0).sum()) / max(1, int((A != 0).sum()))
         print(f"# {M}x{K} at {sp} %: Tiled-CSL {items.nbytes / 1e6:.1f} MB; 2:4 records {packed.nbytes / 1e6:.1f} MB + "
               f"residual {items2.nbytes / 1e6:.1f} MB ({100 * share:.1f} % of the kept values)", flush=True)
         c = args.copies
         d_items, d_offs = [up(items) for _ in range(c)], [up(offs) for _ in range(c)]
         d_p, d_i2, d_o2 = [up(packed) for _ in range(c)], [up(items2) for _ in range(c)], [up(offs2) for _ in range(c)]
+        d_w, d_wo = [up(words) for _ in range(c)], [up(woffs) for _ in range(c)]
         first = True
         for N in [int(x) for x in args.n.split(",")]:
             B = up(G.synth_activations(N, K, seed=1))
@@ -84,9 +87,14 @@ def main():
             t_h = time_us(lambda i: G.HeteroSparse_SpMM_API(st, d_p[i % c], d_i2[i % c], d_o2[i % c], B, C, M, N, K, W, s1, S2))
             t_2 = time_us(lambda i: G.HeteroSparse_SpMM_API(st, d_p[i % c], d_i2[i % c], d_o2[i % c], B, C, M, N, K, W, s1, S2,
                                                            G.HETERO_FLAG_TWO_STREAMS))
+            t_f = float("nan")
+            if longest <= G.HETERO_FUSED_MAX_LIST:
+                t_f = time_us(lambda i: G.HeteroSparse_Fused_SpMM_API(st, d_p[i % c], d_w[i % c], d_wo[i % c], longest, B, C, M, N, K,
+                                                                      W, s1))
             print(f"sparsity {sp} N={N:2d}: csl {t_csl:6.1f} us (Split_K {s0}) | a1 {t_a1:6.1f} us (Split_K {s1}, "
-                  f"{packed.nbytes / t_a1 / 1e6:.2f} TB/s) | hybrid {t_h:6.1f} us (residual Split_K {S2}) | 2-str {t_2:6.1f} us", flush=True)
-        del d_items, d_offs, d_p, d_i2, d_o2
+                  f"{packed.nbytes / t_a1 / 1e6:.2f} TB/s) | hybrid {t_h:6.1f} us (residual Split_K {S2}) | 2-str {t_2:6.1f} us | "
+                  f"fused {t_f:6.1f} us ({(packed.nbytes + words.nbytes) / t_f / 1e6:.2f} TB/s, longest list {longest})", flush=True)
+        del d_items, d_offs, d_p, d_i2, d_o2, d_w, d_wo
         torch.cuda.empty_cache()
 
 

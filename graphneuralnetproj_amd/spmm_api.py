@@ -59,6 +59,8 @@ EXPORTED_SYMBOLS = (
     "HeteroSparse_SuggestSplitK",
     "HeteroSparse_A1_Partials",
     "HeteroSparse_DeviceSplitPack",
+    "HeteroSparse_PackA2",
+    "HeteroSparse_Fused_SpMM_API",
 )
 
 
@@ -170,6 +172,12 @@ def load_library():
     lib.HeteroSparse_DeviceSplitPack.restype = ctypes.c_int
     lib.HeteroSparse_DeviceSplitPack.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
                                                  ctypes.c_void_p, ctypes.c_void_p]
+    lib.HeteroSparse_PackA2.restype = ctypes.c_int
+    lib.HeteroSparse_PackA2.argtypes = [_u16p, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.POINTER(ctypes.c_uint32)),
+                                        ctypes.POINTER(ctypes.POINTER(ctypes.c_int)), ctypes.POINTER(ctypes.c_int)]
+    lib.HeteroSparse_Fused_SpMM_API.restype = ctypes.c_int
+    lib.HeteroSparse_Fused_SpMM_API.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] + [ctypes.c_void_p] * 2 + [ctypes.c_int] * 3 + [
+        ctypes.c_void_p, ctypes.c_int]
     lib.HeteroSparse_A1_Partials.restype = ctypes.c_int
     lib.HeteroSparse_A1_Partials.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 7
     _lib = lib
@@ -427,6 +435,45 @@ def HeteroSparse_SpMM_API(stream, Packed_A1, Compressed_A2, TileOffsets_A2, B, C
                                    _ptr(Reduction_Workspace), Split_K_A1, Split_K_A2, Flags)
     if rc != 0:
         raise SpMMError("HeteroSparse_SpMM_API", rc, lib.SpMM_GetErrorString(rc).decode())
+    return rc
+
+
+HETERO_FUSED_MAX_LIST = 256
+
+
+def HeteroSparse_PackA2(A2_h, M=None, K=None):
+    """Residual lists for HeteroSparse_Fused_SpMM_API -> (words uint32[NNZ + 64], offsets int32, longest list)."""
+    a = _bits(A2_h)
+    if M is None or K is None:
+        M, K = a.shape
+    lib = load_library()
+    words = ctypes.POINTER(ctypes.c_uint32)()
+    offsets = ctypes.POINTER(ctypes.c_int)()
+    longest = ctypes.c_int(0)
+    n = lib.HeteroSparse_PackA2(a.ctypes.data_as(_u16p), M, K, ctypes.byref(words), ctypes.byref(offsets),
+                                ctypes.byref(longest))
+    if n < 0:
+        raise SpMMError("HeteroSparse_PackA2", n)
+    try:
+        offs = np.ctypeslib.as_array(offsets, shape=(n,)).copy()
+        w = np.ctypeslib.as_array(words, shape=(int(offs[-1]) + 64,)).copy()
+    finally:
+        lib.SpMM_FreeHost(words)
+        lib.SpMM_FreeHost(offsets)
+    return w, offs, int(longest.value)
+
+
+def HeteroSparse_Fused_SpMM_API(stream, Packed_A1, A2_Words, A2_Offsets, LongestList, B, C, M_Global, N_Global, K_Global,
+                                Reduction_Workspace, Split_K):
+    """Enqueue C = A1*B + A2*B as one launch (A1 as 2:4 records, A2 as residual lists) on `stream`."""
+    lib = load_library()
+    if stream is not None and not isinstance(stream, int):
+        stream = stream.cuda_stream
+    rc = lib.HeteroSparse_Fused_SpMM_API(ctypes.c_void_p(stream) if stream else None, _ptr(Packed_A1), _ptr(A2_Words),
+                                         _ptr(A2_Offsets), LongestList, _ptr(B), _ptr(C), M_Global, N_Global, K_Global,
+                                         _ptr(Reduction_Workspace), Split_K)
+    if rc != 0:
+        raise SpMMError("HeteroSparse_Fused_SpMM_API", rc, lib.SpMM_GetErrorString(rc).decode())
     return rc
 
 

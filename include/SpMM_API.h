@@ -359,6 +359,36 @@ SPMM_EXPORT int HeteroSparse_SuggestSplitK(int M_Global, int N_Global, int K_Glo
 SPMM_EXPORT int HeteroSparse_A1_Partials(void* stream, const void* Packed_A1, const void* B, void* Partials, int M_Global,
                                          int N_Global, int K_Global, int Split_K, int RowBlocks, int Waves, int ShareB);
 
+/*
+ * Both parts in one launch.  The reference multiplies the residual with a kernel of its own on a
+ * second stream (kernel_benchmark/FSP_Batch8.h:129-206, launched at
+ * kernel_benchmark/spmm_test.cu:462-560); here the 2:4 kernel can take the residual along: every
+ * wave scatters the residual values of its 16 x 128 blocks into a dense image in LDS and multiplies
+ * that on the ordinary matrix cores, against the activation tile and into the accumulators that the
+ * 2:4 part uses, so the activations are read once and nothing is added up afterwards.
+ *
+ * HeteroSparse_PackA2: the residual in the form that launch reads, from row-major A2_h (M x K fp16
+ * bit patterns in host memory, M % 128 == 0, K % 128 == 0): *Words (fp16 value | position << 16, one
+ * list per 16 x 128 block, 4 bytes per kept value) and *Offsets (list i = words Offsets[i] ..
+ * Offsets[i + 1]), both malloc'ed, caller frees; *LongestList = the longest list's length.  *Words
+ * holds Offsets[last] + 64 words (copy them all to the device).  Returns the number of offsets,
+ * (M / 16) * (K / 128) + 1, or -1 bad shape, -2 out of memory, -3 null pointer.
+ *
+ * HeteroSparse_Fused_SpMM_API: C = A1*B + A2*B, one kernel (plus the reduction kernel when
+ * Split_K > 1: Reduction_Workspace then holds Split_K*M*N fp16 values; HeteroSparse_SuggestSplitK).
+ * Device pointers; B[N][K], C[N][M] as for SpMM_SplitK_API.  LongestList as HeteroSparse_PackA2 gave
+ * it, at most HETERO_FUSED_MAX_LIST (uniform sparsity of 50 % and more stays below; a matrix with
+ * denser rows has longer lists and goes through HeteroSparse_SpMM_API instead).  Returns a
+ * hipError_t value: hipErrorUnknown for N outside {8, 16, 32, 64}; hipErrorInvalidValue for M % 128,
+ * K % 128, an empty batch, a list too long, a missing pointer.  Only enqueues work on `stream`.
+ */
+#define HETERO_FUSED_MAX_LIST 256
+SPMM_EXPORT int HeteroSparse_PackA2(const uint16_t* A2_h, int M_Global, int K_Global, uint32_t** Words, int** Offsets,
+                                    int* LongestList);
+SPMM_EXPORT int HeteroSparse_Fused_SpMM_API(void* stream, const void* Packed_A1, const void* A2_Words, const int* A2_Offsets,
+                                            int LongestList, const void* B, void* C, int M_Global, int N_Global,
+                                            int K_Global, void* Reduction_Workspace, int Split_K);
+
 #ifdef __cplusplus
 }
 #endif

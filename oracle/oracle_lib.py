@@ -174,6 +174,31 @@ def a24_unpack(packed, M, K):
     return out.view(np.float16)
 
 
+def residual_unpack(words, offsets, M, K):
+    """Dense fp16 M x K matrix held by residual lists (the build's own format for the launch that
+    multiplies the 2:4 part and the residual together; the reference keeps its residual in a
+    CSR-like form for kernel_benchmark/FSP_Batch8.h:129-206).  List i belongs to the record of the
+    same number, ((rb // 8) * units + u) * 8 + rb % 8 for row block rb and unit u; a word is
+    value | address << 16 with address = r * 256 + (((c // 8) ^ r) << 4) + (c % 8) * 2 for row r and
+    column c of the 16 x 128 block.  Raises on an address twice in one list or out of range."""
+    words = np.ascontiguousarray(words, dtype=np.uint32)
+    offsets = np.ascontiguousarray(offsets, dtype=np.int64)
+    units = K // 128
+    assert offsets.size == (M // 16) * units + 1 and offsets[0] == 0 and (np.diff(offsets) >= 0).all()
+    out = np.zeros((M, K), dtype=np.uint16)
+    for rb in range(M // 16):
+        for u in range(units):
+            i = ((rb // 8) * units + u) * 8 + rb % 8
+            lst = words[offsets[i]:offsets[i + 1]]
+            addr = (lst >> 16).astype(np.int64)
+            if addr.size and (addr.max() >= 4096 or (addr & 1).any() or np.unique(addr).size != addr.size):
+                raise ValueError(f"bad addresses in list {i}")
+            r = addr >> 8
+            c = ((((addr >> 4) & 15) ^ r) << 3) + ((addr & 15) >> 1)
+            out[rb * 16 + r, u * 128 + c] = (lst & 0xFFFF).astype(np.uint16)
+    return out.view(np.float16)
+
+
 # ----------------------------------------------------------------------------
 # the reference's own encoder, where oracle/_ref was built
 

@@ -306,3 +306,186 @@ def test_hybrid_with_row_sharing_residual_launch(spmm, oracle, N):
     B = spmm.synth_activations(N, K, seed=72)
     C = run_hybrid(spmm, packed, items, offsets, B, M, N, K, s1, s2)
     assert_close(C, oracle.gemm_f32(A, B))
+
+
+# ---------------------------------------------------------------------------------------------
+# both parts in one launch
+
+
+def run_fused(spmm, packed, words, offs, longest, B, M, N, K, split_k):
+    torch = _torch()
+    d_p, d_B, d_w, d_o = _dev(packed), _dev(B), _dev(words), _dev(offs)
+    d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device="cuda:0")
+    d_W = torch.full((max(split_k, 1), N, M), float("nan"), dtype=torch.float16, device="cuda:0")
+    print(f"[gpu case] fused M={M} N={N} K={K} split_k={split_k} longest={longest}", flush=True)
+    spmm.HeteroSparse_Fused_SpMM_API(torch.cuda.current_stream(), d_p, d_w, d_o, longest, d_B, d_C, M, N, K, d_W, split_k)
+    torch.cuda.synchronize()
+    return d_C.cpu().numpy()
+
+
+def test_fused_layout_one_hot(spmm, oracle):
+    """Pins rows, columns and tokens of both parts at once: distinct exactly representable integers,
+    one-hot activations, so C[n, m] must equal A[m, k_n] exactly whichever part holds that element."""
+    M, K, N = 256, 384, 16
+    rng = np.random.default_rng(4)
+    A = np.zeros((M, K), dtype=np.float16)
+    mask = rng.random((M, K)) < 0.45
+    vals = (np.arange(M * K).reshape(M, K) % 1999 + 1).astype(np.float16)
+    A[mask] = vals[mask]
+    A1, A2 = oracle.decompose(A)
+    assert np.count_nonzero(A2) > 1000
+    packed = spmm.HeteroSparse_PackA1(A1)
+    words, offs, longest = spmm.HeteroSparse_PackA2(A2)
+    for trial in range(4):
+        ks = rng.permutation(K)[:N]
+        B = np.zeros((N, K), dtype=np.float16)
+        B[np.arange(N), ks] = 1.0
+        C = run_fused(spmm, packed, words, offs, longest, B, M, N, K, 1)
+        assert np.array_equal(C.view(np.uint16), A[:, ks].T.view(np.uint16))
+
+
+@pytest.mark.parametrize("sparsity", [0.5, 0.6, 0.7, 0.8, 0.95])
+@pytest.mark.parametrize("N", [8, 16, 32, 64])
+@pytest.mark.parametrize("M", [384, 512])
+def test_fused_vs_oracle(spmm, oracle, sparsity, N, M):
+    """One to four loads per list (50 % ... 95 % sparsity), four waves (384 rows) and eight (512 rows,
+    once the split gives enough workgroups), nine units split one, two and three ways."""
+    K = 1152
+    A = spmm.synth_weights(M, K, sparsity, False, seed=int(sparsity * 100) + N)
+    B = spmm.synth_activations(N, K, seed=5)
+    A1, A2 = spmm.HeteroSparse_Decompose(A)
+    packed = spmm.HeteroSparse_PackA1(A1)
+    words, offs, longest = spmm.HeteroSparse_PackA2(A2)
+    ref = oracle.gemm_f32(A, B)
+    for split_k in (1, 2, 3):
+        C = run_fused(spmm, packed, words, offs, longest, B, M, N, K, split_k)
+        assert_close(C, ref)
+
+
+@pytest.mark.parametrize("N", [16, 64])
+def test_fused_eight_waves_and_empty_lists(spmm, oracle, N):
+    """49152 rows in workgroups of eight waves (192 of them > 160); rows 0..255 have no residual at
+    all (empty lists at the start), one record's list is the only one of its row block."""
+    M, K = 49152, 256
+    A = spmm.synth_weights(M, K, 0.6, False, seed=N)
+    A[:256] = np.where(np.arange(K) % 4 < 2, A[:256], 0)   # two of four everywhere: nothing left over
+    A[4096:4112, 128:] = np.where(np.arange(128) % 4 < 2, A[4096:4112, 128:], 0)
+    B = spmm.synth_activations(N, K, seed=8)
+    A1, A2 = spmm.HeteroSparse_Decompose(A)
+    assert not A2[:256].any() and not A2[4096:4112, 128:].any()
+    packed = spmm.HeteroSparse_PackA1(A1)
+    words, offs, longest = spmm.HeteroSparse_PackA2(A2)
+    C = run_fused(spmm, packed, words, offs, longest, B, M, N, K, 1)
+    rows = np.r_[0:512, 4000:4200, np.sort(np.random.default_rng(2).choice(M, 1024, replace=False))]
+    assert_close(C[:, rows], oracle.gemm_f32(np.ascontiguousarray(A[rows]), B))
+
+
+def test_fused_without_any_residual(spmm, oracle):
+    M, K, N = 256, 512, 16
+    A, _ = spmm.HeteroSparse_Decompose(spmm.synth_weights(M, K, 0.5, False, seed=10))
+    B = spmm.synth_activations(N, K, seed=6)
+    A1, A2 = spmm.HeteroSparse_Decompose(A)
+    assert not A2.any()
+    words, offs, longest = spmm.HeteroSparse_PackA2(A2)
+    assert longest == 0 and offs[-1] == 0
+    C = run_fused(spmm, spmm.HeteroSparse_PackA1(A1), words, offs, longest, B, M, N, K, 2)
+    assert_close(C, oracle.gemm_f32(A, B))
+
+
+def test_fused_rejects(spmm):
+    torch = _torch()
+    d = torch.zeros(1 << 12, dtype=torch.int32, device="cuda:0")
+    ok = dict(M=256, N=16, K=512, longest=10, s=1)
+    for bad in (dict(M=200), dict(K=576), dict(N=24), dict(s=5), dict(longest=spmm.HETERO_FUSED_MAX_LIST + 1), dict(longest=-1)):
+        a = dict(ok)
+        a.update(bad)
+        with pytest.raises(spmm.SpMMError):
+            spmm.HeteroSparse_Fused_SpMM_API(None, d, d, d, a["longest"], d, d, a["M"], a["N"], a["K"], d, a["s"])
+    with pytest.raises(spmm.SpMMError):
+        spmm.HeteroSparse_Fused_SpMM_API(None, d, None, d, 10, d, d, 256, 16, 512, d, 1)
+    with pytest.raises(spmm.SpMMError):  # a split needs the workspace
+        spmm.HeteroSparse_Fused_SpMM_API(None, d, d, d, 10, d, d, 256, 16, 512, None, 2)
+
+
+def test_fused_row_skewed_weight_has_lists_too_long(spmm):
+    """Beta(2, 8) row densities leave blocks with more than 256 residual values: the packer reports
+    it and the one-launch entry refuses; such a weight goes through HeteroSparse_SpMM_API."""
+    torch = _torch()
+    M, K = 1024, 1024
+    A = spmm.synth_weights(M, K, 0.5, True, seed=3)
+    _, A2 = spmm.HeteroSparse_Decompose(A)
+    words, offs, longest = spmm.HeteroSparse_PackA2(A2)
+    assert longest > spmm.HETERO_FUSED_MAX_LIST
+    d = torch.zeros(1 << 12, dtype=torch.int32, device="cuda:0")
+    with pytest.raises(spmm.SpMMError):
+        spmm.HeteroSparse_Fused_SpMM_API(None, d, d, d, longest, d, d, M, 16, K, d, 1)
+
+
+def test_fused_full_size_sampled_rows(spmm, oracle):
+    """OPT-30B FFN1 at 60 % sparsity, N = 16 and 64: sampled rows against the oracle, the whole
+    result against the two-kernel path (same products, other summation order), and linearity."""
+    M, K = 28672, 7168
+    A = spmm.synth_weights(M, K, 0.6, False, seed=22)
+    A1, A2 = spmm.HeteroSparse_Decompose(A)
+    packed = spmm.HeteroSparse_PackA1(A1)
+    words, offs, longest = spmm.HeteroSparse_PackA2(A2)
+    items, offsets = spmm.InitSparseMatrixA_API(A2)
+    rows = np.sort(np.random.default_rng(0).choice(M, 384, replace=False))
+    Asub = np.ascontiguousarray(A[rows])
+    for N in (16, 64):
+        B1 = spmm.synth_activations(N, K, seed=1)
+        B2 = spmm.synth_activations(N, K, seed=2)
+        s = spmm.HeteroSparse_SuggestSplitK(M, N, K)
+        C1 = run_fused(spmm, packed, words, offs, longest, B1, M, N, K, s)
+        assert_close(C1[:, rows], oracle.gemm_f32(Asub, B1))
+        two = run_hybrid(spmm, packed, items, offsets, B1, M, N, K, s, spmm.SpMM_SuggestSplitK(M, N, K))
+        assert np.isfinite(C1).all()
+        diff = np.abs(C1.astype(np.float32) - two.astype(np.float32))
+        assert (diff <= 2e-2 + 2e-2 * np.abs(two.astype(np.float32))).all()
+        Bs = (B1.astype(np.float32) * 0.5 + B2.astype(np.float32) * 0.5).astype(np.float16)
+        exact = np.array_equal(Bs.astype(np.float32), B1.astype(np.float32) * 0.5 + B2.astype(np.float32) * 0.5)
+        C2 = run_fused(spmm, packed, words, offs, longest, B2, M, N, K, s)
+        Cs = run_fused(spmm, packed, words, offs, longest, Bs, M, N, K, s)
+        lin = 0.5 * C1.astype(np.float32) + 0.5 * C2.astype(np.float32)
+        tol = 2e-2 if exact else 4e-2
+        assert (np.abs(Cs.astype(np.float32) - lin) <= tol + tol * np.abs(lin)).all()
+
+
+def test_fused_hip_graph_replays_match_eager(spmm, oracle):
+    torch = _torch()
+    M, K, N = 1024, 1024, 16
+    A = spmm.synth_weights(M, K, 0.6, False, seed=33)
+    A1, A2 = spmm.HeteroSparse_Decompose(A)
+    d_p = _dev(spmm.HeteroSparse_PackA1(A1))
+    words, offs, longest = spmm.HeteroSparse_PackA2(A2)
+    d_w, d_o = _dev(words), _dev(offs)
+    Bh = spmm.synth_activations(N, K, seed=34)
+    d_B = _dev(Bh)
+    d_C = torch.zeros((N, M), dtype=torch.float16, device="cuda:0")
+    d_W = torch.zeros((2, N, M), dtype=torch.float16, device="cuda:0")
+
+    def call(stream):
+        spmm.HeteroSparse_Fused_SpMM_API(stream, d_p, d_w, d_o, longest, d_B, d_C, M, N, K, d_W, 2)
+
+    print("[gpu case] graph capture of the one-launch 2:4 + residual call", flush=True)
+    call(torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    want = d_C.clone()
+    assert_close(want.cpu().numpy(), oracle.gemm_f32(A, Bh))
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            call(torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    for rep in range(3):
+        d_C.zero_()
+        d_W.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(d_C, want), f"replay {rep} differs from the eager result"
+        d_C.zero_()
+        call(torch.cuda.current_stream())
+        torch.cuda.synchronize()
+        assert torch.equal(d_C, want)
+

@@ -189,3 +189,76 @@ def test_record_order_groups_eight_row_blocks(spmm, oracle):
         for u in range(units):
             assert first[((rb // 8) * units + u) * 8 + rb % 8] == H(rb * units + u + 1)
     assert np.array_equal(oracle.a24_unpack(packed.reshape(-1), M, K).view(np.uint16), A.view(np.uint16))
+
+
+def test_oracle_residual_unpack_reads_hand_built_lists(oracle):
+    """Two words written by hand from the format's definition: row 5, column 77 of block 9 / unit 1
+    and row 0, column 0 of block 0 / unit 0 of a 256 x 256 matrix."""
+    M, K, units = 256, 256, 2
+    offs = np.zeros((M // 16) * units + 1, dtype=np.int32)
+    first = ((0 // 8) * units + 0) * 8 + 0
+    second = ((9 // 8) * units + 1) * 8 + 9 % 8
+    offs[first + 1:] += 1
+    offs[second + 1:] += 1
+    r, c = 5, 77
+    addr = r * 256 + (((c // 8) ^ r) << 4) + (c % 8) * 2
+    assert addr == 5 * 256 + ((9 ^ 5) << 4) + 10
+    words = np.array([0x3C00 | 0 << 16, 0x4000 | addr << 16], dtype=np.uint32)  # 1.0 and 2.0
+    A = oracle.residual_unpack(words, offs, M, K)
+    want = np.zeros((M, K), dtype=H)
+    want[0, 0] = 1
+    want[9 * 16 + 5, 128 + 77] = 2
+    assert np.array_equal(A.view(np.uint16), want.view(np.uint16))
+    with pytest.raises(ValueError):  # the same place twice
+        oracle.residual_unpack(np.array([0x3C00, 0x3C00], dtype=np.uint32), np.minimum(np.arange(offs.size), 2).astype(np.int32) * 0
+                               + np.r_[0, np.full(offs.size - 1, 2)].astype(np.int32), M, K)
+
+
+@pytest.mark.parametrize("M,K,keep", [(128, 128, 0.5), (256, 640, 0.4), (384, 1024, 0.2), (128, 256, 0.0), (128, 128, 1.0)])
+def test_residual_lists_round_trip(spmm, oracle, M, K, keep):
+    rng = np.random.default_rng(M + K + 1)
+    A = _rand_sparse(rng, M, K, keep)
+    A.view(np.uint16)[0, :8] = [0x8000, 0x7E00, 0x0001, 0x3C00, 0xFC00, 0x8001, 0, 0x7C00]  # -0, NaN, denormals, infinities
+    _, A2 = oracle.decompose(A)
+    words, offs, longest = spmm.HeteroSparse_PackA2(A2)
+    units = K // 128
+    assert offs.size == (M // 16) * units + 1 and offs[0] == 0
+    assert words.size == offs[-1] + 64 and not words[offs[-1]:].any()  # the padding the kernel may read
+    lengths = np.diff(offs)
+    assert longest == (lengths.max() if lengths.size else 0)
+    assert offs[-1] == np.count_nonzero(A2.view(np.uint16) & 0x7FFF)   # one word per kept value, -0 is not one
+    back = oracle.residual_unpack(words[:offs[-1]], offs, M, K)
+    want = A2.view(np.uint16).copy()
+    want[(want & 0x7FFF) == 0] = 0
+    assert np.array_equal(back.view(np.uint16), want)
+    # Every round of 64 words spreads over the banks: with three or more rounds no round holds more of
+    # a bank than an even split over the full rounds, and in all the serialised passes (the fullest
+    # bank of every round, summed) are fewer than in row-major order.
+    def passes(lst):
+        bank = ((lst >> 16) >> 2) & 63
+        return sum(np.bincount(bank[r:r + 64], minlength=64).max() for r in range(0, lst.size, 64))
+
+    ordered = plain = 0
+    for i in range(offs.size - 1):
+        lst = words[offs[i]:offs[i + 1]]
+        rounds = -(-lst.size // 64)
+        if rounds <= 1:
+            continue
+        bank = ((lst >> 16) >> 2) & 63
+        total = np.bincount(bank, minlength=64)
+        if rounds >= 3:
+            for r in range(rounds):
+                assert (np.bincount(bank[r * 64:(r + 1) * 64], minlength=64) <= -(-total // (rounds - 1))).all()
+        ordered += passes(lst)
+        plain += passes(np.sort(lst >> 16) << 16)
+    assert ordered <= plain
+    if keep in (0.4, 0.5):  # lists of two to four rounds, banks unevenly filled
+        assert ordered < 0.9 * plain
+
+
+def test_residual_lists_reject_bad_shapes(spmm):
+    for shape in ((128, 64), (64, 128), (200, 128)):
+        with pytest.raises(spmm.SpMMError) as e:
+            spmm.HeteroSparse_PackA2(np.zeros(shape, dtype=H))
+        assert e.value.code == -1
+
