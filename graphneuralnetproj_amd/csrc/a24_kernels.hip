@@ -319,16 +319,20 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
     const long list0 = ((long)(block0 / kGroupBlocks) * units) * kGroupBlocks + block0 % kGroupBlocks;
     const int* const off_lane = offsets + list0 + (lane <= RB ? lane : RB);
     unsigned char* const image = tile + 2 * kBuf + wave * kImageBytes;
-    // o[0..RB]: the offsets of `unit`'s lists, the same in every lane
-    auto issue_unit = [&](UnitRegs& x, int unit, int unit_after, const int (&o)[RB + 1]) {
+    // A unit's loads: the offsets of the unit after it, its activation chunks (needed first), its
+    // records, and (issue_words; o[0..RB] = the offsets of the unit's lists, the same in every lane)
+    // its residual words.
+    auto issue_head = [&](UnitRegs& x, int unit, int unit_after) {
         if constexpr (RL > 0)
             asm volatile("global_load_dword %0, %1, off" : "=v"(x.next) : "v"(off_lane + (size_t)unit_after * kGroupBlocks));
 #pragma unroll
-        for (int i = 0; i < CH; i++)  // activation chunks before the records: they are needed first
+        for (int i = 0; i < CH; i++)
             x.stage[i] = issue_b(src[i] + (size_t)unit * 128);
 #pragma unroll
         for (int r = 0; r < RB; r++)
             x.a[r] = issue_a(rec[r] + (size_t)unit * kUnitStride + lane * 16, rec[r] + (size_t)unit * kUnitStride + lane * 4);
+    };
+    auto issue_words = [&](UnitRegs& x, const int (&o)[RB + 1]) {
         if constexpr (RL > 0) {
 #pragma unroll
             for (int r = 0; r < RB; r++) {
@@ -343,6 +347,10 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
                 }
             }
         }
+    };
+    auto issue_unit = [&](UnitRegs& x, int unit, int unit_after, const int (&o)[RB + 1]) {
+        issue_head(x, unit, unit_after);
+        issue_words(x, o);
     };
     // The offsets that a unit's `next` load brought, once it has landed.
     auto offsets_from = [&](UnitRegs& x, int (&o)[RB + 1]) {
@@ -435,23 +443,27 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
         auto ahead = [&](int d) { return u + d < last ? u + d : last; };
         int o[RB + 1] = {};
         if constexpr (RL > 0) {
-            // the image starts out clear; the first two units' offsets are fetched by themselves
-            for (int i = lane * 16; i < kImageBytes; i += kWave * 16)
-                *reinterpret_cast<u32x4*>(image + i) = u32x4{0u, 0u, 0u, 0u};
+            // The first two units' offsets are fetched by themselves, and their records and
+            // activation chunks go out before those offsets are back; their words follow.  The
+            // queue of the first phase is therefore: records(u), unit u + 1's head, words(u), words(u + 1).
             int first, second;
             asm volatile("global_load_dword %0, %1, off" : "=v"(first) : "v"(off_lane + (size_t)u * kGroupBlocks));
             asm volatile("global_load_dword %0, %1, off" : "=v"(second) : "v"(off_lane + (size_t)ahead(1) * kGroupBlocks));
-            wait_loads<0>();
+            issue_head(x[0], u, ahead(1));
+            issue_head(x[1], ahead(1), ahead(2));
+            for (int i = lane * 16; i < kImageBytes; i += kWave * 16)  // the image starts out clear
+                *reinterpret_cast<u32x4*>(image + i) = u32x4{0u, 0u, 0u, 0u};
+            wait_loads<2 * (kLoadsHead + CH + 3 * RB)>();
             settle(first);
             settle(second);
 #pragma unroll
             for (int j = 0; j <= RB; j++)
                 o[j] = __builtin_amdgcn_readlane(first, j);
-            issue_unit(x[0], u, ahead(1), o);
+            issue_words(x[0], o);
 #pragma unroll
             for (int j = 0; j <= RB; j++)
                 o[j] = __builtin_amdgcn_readlane(second, j);
-            issue_unit(x[1], ahead(1), ahead(2), o);
+            issue_words(x[1], o);
         } else {
             issue_unit(x[0], u, u, o);
             issue_unit(x[1], ahead(1), u, o);
@@ -459,10 +471,13 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
         wait_loads<kLoadsA + kLoadsHead + CH + kLoadsA>();  // the first tile
         store_b(x[0], 0);
         __syncthreads();
-        auto phase = [&](auto kc) {  // unit u, whose registers are set kc
+        auto phase = [&](auto kc, auto is_first) {  // unit u, whose registers are set kc
             constexpr int k = decltype(kc)::value;
             const int buf = (u - u0) & 1;
-            wait_loads<kLoadsA>();
+            if constexpr (RL > 0 && decltype(is_first)::value)
+                wait_loads<RL * RB>();  // only words(u + 1) are younger than what the first phase needs
+            else
+                wait_loads<kLoadsA>();
             landed(x[k]);
             store_b(x[(k + 1) % 3], buf ^ 1);
             int o2[RB + 1] = {};
@@ -474,17 +489,19 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
         };
         // Whole rounds of three units, then the rest: no exit from inside a round, so that every
         // path through the loop carries the same loads in the same registers.
-        const int units_here = u1 - u0;
-        for (int round = units_here / 3; round > 0; round--) {
-            phase(std::integral_constant<int, 0>{});
-            phase(std::integral_constant<int, 1>{});
-            phase(std::integral_constant<int, 2>{});
+        using std::integral_constant;
+        const int units_after_first = u1 - u0 - 1;
+        phase(integral_constant<int, 0>{}, integral_constant<bool, true>{});
+        for (int round = units_after_first / 3; round > 0; round--) {
+            phase(integral_constant<int, 1>{}, integral_constant<bool, false>{});
+            phase(integral_constant<int, 2>{}, integral_constant<bool, false>{});
+            phase(integral_constant<int, 0>{}, integral_constant<bool, false>{});
         }
-        const int rest = units_here % 3;
+        const int rest = units_after_first % 3;
         if (rest >= 1) {
-            phase(std::integral_constant<int, 0>{});
+            phase(integral_constant<int, 1>{}, integral_constant<bool, false>{});
             if (rest >= 2)
-                phase(std::integral_constant<int, 1>{});
+                phase(integral_constant<int, 2>{}, integral_constant<bool, false>{});
         }
         // the repeated loads of the last phases are still on their way into registers that the
         // stores below may reuse
