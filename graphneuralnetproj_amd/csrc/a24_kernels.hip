@@ -567,9 +567,9 @@ int launch_shared_b_nt(hipStream_t s, const void* packed, const void* B, void* o
         return launch_shared_b<NT, RB_, W_, RL_>(s, packed, B, out, M, N, K, split_k, ldb, ldo, slab, words, offsets);
     A24_CASE(2, 4, 0) A24_CASE(2, 8, 0)
     A24_CASE(2, 4, 1) A24_CASE(2, 8, 1) A24_CASE(2, 4, 2) A24_CASE(2, 8, 2) A24_CASE(2, 4, 3) A24_CASE(2, 8, 3)
-    A24_CASE(2, 4, 4)
+    A24_CASE(2, 4, 4) A24_CASE(2, 4, 5)
     if constexpr (NT <= 2) {
-        A24_CASE(2, 8, 4)  // with 64 tokens it would not fit 256 registers  // three record sets of four row blocks do not fit the registers beside 64 tokens
+        A24_CASE(2, 8, 4) A24_CASE(2, 8, 5)  // with 64 tokens they would not fit 256 registers  // three record sets of four row blocks do not fit the registers beside 64 tokens
         A24_CASE(4, 2, 0) A24_CASE(4, 4, 0) A24_CASE(4, 8, 0)
     }
 #undef A24_CASE

@@ -480,49 +480,48 @@ struct A24Plan {
     int share_b = 0;  // 0: the waves of a workgroup split K and add up; 1: they split rows and share the activation tile in LDS
 };
 
+// Waves per workgroup for a given split: eight (256 rows) where that many workgroups still fill
+// the chip, else four (two such workgroups share a compute unit).
+int a24_waves_for(int M, int split_k)
+{
+    return (M % 256 == 0 && static_cast<long>(M / 256) * split_k > 160) ? 8 : 4;
+}
+
 A24Plan a24_default_plan(int M, int N, int K)
 {
-    // From sweeps over the OPT-30B and OPT-66B shapes (N = 16 and 64): waves that own two row blocks
-    // each and share the activation tile through LDS, eight of them per workgroup where the rows
-    // allow (256 rows, two groups of records), else four; and the split-K with the least estimated
-    // time: rounds of up to 256 workgroups, each round streaming its share of the records at one
-    // compute unit's rate plus a fixed cost, and a small cost per slab.  That picks the counts the
-    // sweeps found fastest: just under 256 workgroups (216 to 252) where the rows allow, else e.g.
-    // 432 rather than 144 or 288.
-    A24Plan p{2, M % 256 == 0 ? 8 : 4, 1, 1};
-    (void)N;
-    const long groups = M / (16 * p.row_blocks * p.waves);
+    // From sweeps over the OPT-30B and OPT-66B shapes (N = 16 and 64, with and without the residual):
+    // waves that own two row blocks each and share the activation tile through LDS, and the split-K
+    // with the least estimated time for the finished result: rounds of workgroups (256 of eight
+    // waves or 512 of four at a time), each compute unit streaming its share of the records at one
+    // unit's rate plus a fixed cost per round, and the reduction kernel plus a cost per slab once
+    // there is more than one batch.  That picks what the sweeps found fastest: just under 256
+    // workgroups of eight waves or as many of four with half the slabs (FFN1 28672x7168, N = 16:
+    // four waves, one batch, no reduction: 36.0 us against 35.2 + 3 us), else e.g. 432 rather than
+    // 144 or 288.  With 64 tokens eight waves hide the matrix cores' and the LDS's latencies better
+    // (FFN1: 41 us + reduction against 46).
+    A24Plan p{2, 4, 1, 1};
     const int units = K / a24::kUnitCols;
     const double bytes = static_cast<double>(a24::bytes(M, K));
-    constexpr double kUnitBytesPerUs = 25.4e3, kRoundUs = 6.0, kSlabUs = 0.5;
+    constexpr double kUnitBytesPerUs = 25.4e3, kRoundUs = 6.0, kReduceUs = 3.0, kSlabUs = 0.8, kFourWaves64 = 1.15;
     double best = 0.0;
     for (int s = 1; s <= 32 && s <= units; s++) {
         const int per = (units + s - 1) / s;
         if ((s > 1 && per < 2) || static_cast<long>(per) * (s - 1) >= units)
             continue;  // batches of one unit, or an empty last batch
-        const long n = groups * s;
-        const double cost = static_cast<double>((n + 255) / 256) * (bytes / n / kUnitBytesPerUs + kRoundUs) + kSlabUs * s;
+        const int waves = a24_waves_for(M, s);
+        const long n = static_cast<long>(M / (16 * p.row_blocks * waves)) * s;
+        const long at_once = waves == 8 ? 256 : 512;
+        const long rounds = (n + at_once - 1) / at_once;
+        const long per_unit = ((n < at_once ? n : at_once) + 255) / 256;  // workgroups that share a compute unit
+        const double stream = bytes / n * per_unit / kUnitBytesPerUs * (N == 64 && waves == 4 ? kFourWaves64 : 1.0);
+        const double cost = rounds * (stream + kRoundUs) + (s > 1 ? kReduceUs + kSlabUs * s : 0.0);
         if (best == 0.0 || cost < best * 0.999) {
             best = cost;
             p.split_k = s;
+            p.waves = waves;
         }
     }
-    // Half the slabs from half as many waves per workgroup: the same number of workgroups, two of
-    // them on a compute unit, and with an even split of two no reduction kernel at all (FFN1
-    // 28672x7168, N = 16: 36.0 us against 35.2 + 3 us).  With 64 tokens eight waves hide the matrix
-    // cores' and the LDS's latencies better (41 us against 46).
-    if (N <= 32 && p.waves == 8 && p.split_k % 2 == 0) {
-        p.waves = 4;
-        p.split_k /= 2;
-    }
     return p;
-}
-
-// Waves per workgroup for a caller-chosen split: eight (256 rows) where that many workgroups still
-// fill the chip, else four.
-int a24_waves_for(int M, int split_k)
-{
-    return (M % 256 == 0 && static_cast<long>(M / 256) * split_k > 160) ? 8 : 4;
 }
 
 bool a24_shape_ok(int M, int N, int K, int split_k, int row_blocks, int waves, int share_b = 0)
@@ -669,7 +668,7 @@ extern "C" int HeteroSparse_Fused_SpMM_API(void* stream, const void* Packed_A1, 
     const int loads = (LongestList + 63) / 64;
     const long mn = static_cast<long>(M) * N;
     void* out = Split_K == 1 ? C : Reduction_Workspace;
-    const int waves = (N == 64 && loads == 4) ? 4 : a24_waves_for(M, Split_K);  // the former: what fits the registers
+    const int waves = (N == 64 && loads >= 4) ? 4 : a24_waves_for(M, Split_K);  // the former: what fits the registers
     const int rc = a24_launch_spmm(stream, Packed_A1, B, out, M, N, K, Split_K, d.row_blocks, waves, d.share_b, K, M, mn,
                                    loads, A2_Words, A2_Offsets);
     if (rc != 0 || Split_K == 1)

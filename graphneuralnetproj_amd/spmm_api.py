@@ -438,7 +438,7 @@ def HeteroSparse_SpMM_API(stream, Packed_A1, Compressed_A2, TileOffsets_A2, B, C
     return rc
 
 
-HETERO_FUSED_MAX_LIST = 256
+HETERO_FUSED_MAX_LIST = 320
 
 
 def HeteroSparse_PackA2(A2_h, M=None, K=None):

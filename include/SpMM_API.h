@@ -382,7 +382,7 @@ SPMM_EXPORT int HeteroSparse_A1_Partials(void* stream, const void* Packed_A1, co
  * hipError_t value: hipErrorUnknown for N outside {8, 16, 32, 64}; hipErrorInvalidValue for M % 128,
  * K % 128, an empty batch, a list too long, a missing pointer.  Only enqueues work on `stream`.
  */
-#define HETERO_FUSED_MAX_LIST 256
+#define HETERO_FUSED_MAX_LIST 320
 SPMM_EXPORT int HeteroSparse_PackA2(const uint16_t* A2_h, int M_Global, int K_Global, uint32_t** Words, int** Offsets,
                                     int* LongestList);
 SPMM_EXPORT int HeteroSparse_Fused_SpMM_API(void* stream, const void* Packed_A1, const void* A2_Words, const int* A2_Offsets,
