@@ -209,9 +209,79 @@ def sweep(G, lib, torch, dev, sptr, with_stack):
                     "ms": ms, "frac": a_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                     "tflops": 2.0 * M * N * K / (ms * 1e-3) / 1e12})
     cache.clear()
+    for sparsity in (0.6, 0.7):
+        out.append(split_case(G, lib, torch, dev, sptr, "opt30b_ffn1", 16, sparsity))
     if with_stack:
         out.append(stack_step(G, torch, dev))
     return out
+
+
+def split_case(G, lib, torch, dev, sptr, workload, N, sparsity):
+    """The fork's split of a weight into a 2:4 part and a residual, at a sparsity where it can pay:
+    plain Tiled-CSL, the two-kernel call and the one-launch call on the same weight, whole calls
+    between two events, weights rotated over three copies."""
+    M, K = WORKLOADS[workload][:2]
+    A = G.synth_weights(M, K, sparsity, False, seed=1234)
+    A1, A2 = G.HeteroSparse_Decompose(A)
+    items, offsets = G.InitSparseMatrixA_API(A)
+    del A
+    packed = G.HeteroSparse_PackA1(A1)
+    del A1
+    items2, offsets2 = G.InitSparseMatrixA_API(A2)
+    words, list_offsets, longest = G.HeteroSparse_PackA2(A2)
+    del A2
+    copies = 3
+
+    def up(a):
+        a = a.view(np.int32) if a.dtype == np.uint32 else a
+        return [torch.from_numpy(a).to(dev) for _ in range(copies)]
+
+    d = {k: up(v) for k, v in dict(items=items, offs=offsets, packed=packed, items2=items2, offs2=offsets2, words=words,
+                                    lists=list_offsets).items()}
+    p = {k: [ctypes.c_void_p(t.data_ptr()) for t in v] for k, v in d.items()}
+    s_csl = G.SpMM_SuggestSplitK_Bytes(M, N, K, int(offsets[-1]))
+    s_res = G.SpMM_SuggestSplitK(M, N, K)
+    s_a1 = G.HeteroSparse_SuggestSplitK(M, N, K)
+    d_B = torch.from_numpy(G.synth_activations(N, K, seed=4321).view(np.int16)).to(dev)
+    d_C = torch.zeros((N, M), dtype=torch.float16, device=dev)
+    d_W = torch.zeros((s_csl + s_res + s_a1, N, M), dtype=torch.float16, device=dev)
+    p_B, p_C, p_W = (ctypes.c_void_p(t.data_ptr()) for t in (d_B, d_C, d_W))
+
+    def check(rc, what):
+        if rc:
+            raise RuntimeError(f"{what} -> {rc}")
+
+    def csl(i):
+        check(lib.SpMM_SplitK_API(sptr, None, p["items"][i % copies], p["offs"][i % copies], p_B, p_C, M, N, K, p_W, s_csl),
+              "SpMM_SplitK_API")
+
+    def two(i):
+        check(lib.HeteroSparse_SpMM_API(sptr, p["packed"][i % copies], p["items2"][i % copies], p["offs2"][i % copies], p_B, p_C,
+                                        M, N, K, p_W, s_a1, s_res, 0), "HeteroSparse_SpMM_API")
+
+    def one(i):
+        check(lib.HeteroSparse_Fused_SpMM_API(sptr, p["packed"][i % copies], p["words"][i % copies], p["lists"][i % copies], longest,
+                                              p_B, p_C, M, N, K, p_W, s_a1), "HeteroSparse_Fused_SpMM_API")
+
+    res = {}
+    outputs = {}
+    for name, fn in (("tiled_csl", csl), ("two_kernels", two), ("one_launch", one)):
+        if name == "one_launch" and longest > G.HETERO_FUSED_MAX_LIST:
+            res[name] = None
+            continue
+        prewarm(fn, torch, 0.1)
+        res[name] = float(np.median([events_ms(lib, sptr, fn, 100) for _ in range(3)])) / 100
+        torch.cuda.synchronize()
+        outputs[name] = d_C.float().cpu().numpy()
+    ref = outputs["tiled_csl"]
+    agree = all(bool((np.abs(o - ref) <= 2e-2 + 2e-2 * np.abs(ref)).all()) for o in outputs.values())
+    one_bytes = packed.nbytes + 4 * int(list_offsets[-1])
+    best = res["one_launch"] or res["two_kernels"]
+    return {"case": f"ffn1_{int(sparsity * 100)}pct_2to4_plus_residual", "M": M, "K": K, "N": N, "sparsity": sparsity,
+            "tiled_csl_bytes": 16 * int(offsets[-1]), "records_bytes": packed.nbytes, "residual_list_bytes": 4 * int(list_offsets[-1]),
+            "tiled_csl_ms": res["tiled_csl"], "two_kernels_ms": res["two_kernels"], "one_launch_ms": res["one_launch"],
+            "split_k": {"tiled_csl": s_csl, "records": s_a1, "residual": s_res}, "outputs_agree": agree,
+            "ms": best, "frac": one_bytes / (best * 1e-3) / 1e9 / HBM_PEAK_GBPS}
 
 
 def stack_step(G, torch, dev, layers=64, h=9216, N=16, sparsity=0.8):
