@@ -657,20 +657,19 @@ extern "C" int HeteroSparse_Fused_SpMM_API(void* stream, const void* Packed_A1, 
         std::printf("MM_Sparse_API Error: Unsupported N dimension %d!\n", N);  // csrc/SpMM_API.cu:192-193
         return tcsl_error_unknown();
     }
-    const A24Plan d = a24_shape_ok(M, N, K, Split_K, 1, 1) ? a24_default_plan(M, N, K) : A24Plan{1, 1, 1};
+    // two row blocks per wave, activation tile shared through LDS: the one layout that takes the residual along
+    const int loads = (LongestList + 63) / 64;
+    const int waves = (N == 64 && loads >= 4) ? 4 : a24_waves_for(M > 0 ? M : 128, Split_K);  // the former: what fits the registers
     if (!Packed_A1 || !A2_Words || !A2_Offsets || !B || !C || LongestList < 0 || LongestList > HETERO_FUSED_MAX_LIST
-        || !a24_shape_ok(M, N, K, Split_K, d.row_blocks, d.waves, d.share_b) || d.row_blocks != 2 || !d.share_b
-        || (Split_K > 1 && !Reduction_Workspace)) {
+        || !a24_shape_ok(M, N, K, Split_K, 2, waves, 1) || (Split_K > 1 && !Reduction_Workspace)) {
         std::fprintf(stderr, "HeteroSparse_Fused_SpMM_API: unsupported call M=%d N=%d K=%d Split_K=%d LongestList=%d (need M %% 128 == 0, K %% 128 == 0, no empty batch, lists of at most %d words, non-null pointers)\n",
                      M, N, K, Split_K, LongestList, HETERO_FUSED_MAX_LIST);
         return tcsl_error_invalid_value();
     }
-    const int loads = (LongestList + 63) / 64;
     const long mn = static_cast<long>(M) * N;
     void* out = Split_K == 1 ? C : Reduction_Workspace;
-    const int waves = (N == 64 && loads >= 4) ? 4 : a24_waves_for(M, Split_K);  // the former: what fits the registers
-    const int rc = a24_launch_spmm(stream, Packed_A1, B, out, M, N, K, Split_K, d.row_blocks, waves, d.share_b, K, M, mn,
-                                   loads, A2_Words, A2_Offsets);
+    const int rc = a24_launch_spmm(stream, Packed_A1, B, out, M, N, K, Split_K, 2, waves, 1, K, M, mn, loads, A2_Words,
+                                   A2_Offsets);
     if (rc != 0 || Split_K == 1)
         return rc;
     return tcsl_launch_reduce(stream, C, static_cast<uint16_t*>(Reduction_Workspace), mn, 1, mn, Split_K, 0);

@@ -362,6 +362,18 @@ def test_fused_vs_oracle(spmm, oracle, sparsity, N, M):
         assert_close(C, ref)
 
 
+@pytest.mark.parametrize("M,K,split_k", [(128, 128, 1), (128, 384, 3), (256, 256, 2), (640, 512, 1)])
+def test_fused_shortest_batches(spmm, oracle, M, K, split_k):
+    """Batches of a single unit (the pipeline's start and end only) and of two."""
+    N = 32
+    A = spmm.synth_weights(M, K, 0.55, False, seed=M + K)
+    B = spmm.synth_activations(N, K, seed=9)
+    A1, A2 = spmm.HeteroSparse_Decompose(A)
+    words, offs, longest = spmm.HeteroSparse_PackA2(A2)
+    C = run_fused(spmm, spmm.HeteroSparse_PackA1(A1), words, offs, longest, B, M, N, K, split_k)
+    assert_close(C, oracle.gemm_f32(A, B))
+
+
 @pytest.mark.parametrize("N", [16, 64])
 def test_fused_eight_waves_and_empty_lists(spmm, oracle, N):
     """49152 rows in workgroups of eight waves (192 of them > 160); rows 0..255 have no residual at
