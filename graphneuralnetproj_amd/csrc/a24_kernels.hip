@@ -728,6 +728,230 @@ extern "C" int a24_launch_split_pack(void* stream, const void* A, void* packed, 
     return static_cast<int>(hipGetLastError());
 }
 
+// The residual lists (a24_format.h) on the GPU, from the dense residual that the split above
+// leaves in device memory: the same words in the same order as the host's pack_residual
+// (a24_pack.cpp).  Three kernels: count per record, scan, emit.  One wave per record: lane L
+// reads columns 32 * (L % 4) .. + 31 of row L / 4, so lane order is the row-major order that the
+// host collects a list in.
+namespace {
+
+constexpr int kMaxListWords = 16 * 128 / 2;  // a residual holds at most two of every four
+
+__device__ __forceinline__ bool residual_kept(unsigned v)
+{
+    return (v & 0x7fffu) != 0;
+}
+
+__device__ __forceinline__ void record_of_list(long list, int units, long& rb, int& u)
+{
+    const long group = list / (static_cast<long>(units) * kGroupBlocks);
+    const int within = static_cast<int>(list - group * units * kGroupBlocks);
+    u = within / kGroupBlocks;
+    rb = group * kGroupBlocks + within % kGroupBlocks;
+}
+
+typedef unsigned short u16x8v __attribute__((ext_vector_type(8)));
+
+__global__ __launch_bounds__(256) void a24_residual_count_kernel(const uint16_t* __restrict__ A2, int K, int units,
+                                                                 long lists, int* __restrict__ offsets)
+{
+    const long list = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (list >= lists)
+        return;
+    const int L = threadIdx.x & 63;
+    long rb;
+    int u;
+    record_of_list(list, units, rb, u);
+    const uint16_t* src = A2 + (size_t)(rb * 16 + (L >> 2)) * K + (size_t)u * 128 + (L & 3) * 32;
+    int n = 0;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const u16x8v v = *reinterpret_cast<const u16x8v*>(src + q * 8);
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+            n += residual_kept(v[e]) ? 1 : 0;
+    }
+    for (int o = 32; o > 0; o >>= 1)
+        n += __shfl_down(n, o);
+    if (L == 0)
+        offsets[list + 1] = n;
+}
+
+// offsets[1..lists] hold the lists' lengths; turn them into running totals (offsets[0] = 0) and
+// report the longest.  One workgroup.  A total beyond what an int holds gives offsets[lists] = -1.
+__global__ __launch_bounds__(1024) void a24_residual_scan_kernel(int* __restrict__ offsets, long lists,
+                                                                 int* __restrict__ longest)
+{
+    __shared__ long long sums[1024];
+    __shared__ int most[1024];
+    const long chunk = (lists + 1023) / 1024;
+    const long lo = threadIdx.x * chunk, hi = lo + chunk < lists ? lo + chunk : lists;
+    long long s = 0;
+    int m = 0;
+    for (long i = lo; i < hi; i++) {
+        const int n = offsets[i + 1];
+        s += n;
+        m = n > m ? n : m;
+    }
+    sums[threadIdx.x] = s;
+    most[threadIdx.x] = m;
+    __syncthreads();
+    for (int o = 1; o < 1024; o <<= 1) {
+        const long long v = threadIdx.x >= o ? sums[threadIdx.x - o] : 0;
+        const int w = threadIdx.x >= o ? most[threadIdx.x - o] : 0;
+        __syncthreads();
+        sums[threadIdx.x] += v;
+        most[threadIdx.x] = w > most[threadIdx.x] ? w : most[threadIdx.x];
+        __syncthreads();
+    }
+    const bool fits = sums[1023] <= 0x7fffffffLL - 64;
+    long long run = threadIdx.x ? sums[threadIdx.x - 1] : 0;
+    for (long i = lo; i < hi; i++) {
+        run += offsets[i + 1];
+        offsets[i + 1] = fits ? static_cast<int>(run) : (i + 1 == lists ? -1 : 0);
+    }
+    if (threadIdx.x == 0) {
+        offsets[0] = 0;
+        *longest = most[1023];
+    }
+}
+
+// One wave (= one workgroup) per list.
+__global__ __launch_bounds__(64) void a24_residual_emit_kernel(const uint16_t* __restrict__ A2, int K, int units, long lists,
+                                                               const int* __restrict__ offsets, uint32_t* __restrict__ words)
+{
+    __shared__ uint32_t natural[kMaxListWords];  // the list in row-major order, later in its final order
+    __shared__ uint32_t by_bank[kMaxListWords];  // grouped by bank, fullest bank first
+    __shared__ int order[64], count_of[64], start_of[64], used[16], mine[16];
+    const long list = blockIdx.x;
+    const int L = threadIdx.x;
+    long rb;
+    int u;
+    record_of_list(list, units, rb, u);
+    const int row = L >> 2, c0 = (L & 3) * 32;
+    const uint16_t* src = A2 + (size_t)(rb * 16 + row) * K + (size_t)u * 128 + c0;
+    u16x8v v[4];
+    int mine_n = 0;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        v[q] = *reinterpret_cast<const u16x8v*>(src + q * 8);
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+            mine_n += residual_kept(v[q][e]) ? 1 : 0;
+    }
+    int incl = mine_n;  // inclusive scan over the lanes
+    for (int o = 1; o < 64; o <<= 1) {
+        const int t = __shfl_up(incl, o);
+        if (L >= o)
+            incl += t;
+    }
+    const int n = __shfl(incl, 63);
+    const int begin = offsets[list];
+    if (list == lists - 1)  // the padding behind the last list
+        words[(size_t)offsets[lists] + L] = 0;
+    if (n == 0)
+        return;
+    int at = incl - mine_n;
+    const bool in_order = n <= 64;  // one round: the host leaves such a list as collected
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+            if (residual_kept(v[q][e])) {
+                const int c = c0 + q * 8 + e;
+                const uint32_t address = row * 256 + ((((c >> 3) ^ row) & 15) << 4) + (c & 7) * 2;
+                const uint32_t w = v[q][e] | address << 16;
+                if (in_order)
+                    words[(size_t)begin + at] = w;
+                else
+                    natural[at] = w;
+                at++;
+            }
+    if (in_order)
+        return;
+    __syncthreads();
+    // lane b looks after bank b: how many words, where they start among the banks sorted by
+    // (count descending, bank ascending), and its words in collected order
+    auto bank_of = [](uint32_t w) { return static_cast<int>(((w >> 16) >> 2) & 63); };
+    int cnt = 0;
+    for (int i = 0; i < n; i++)
+        cnt += bank_of(natural[i]) == L ? 1 : 0;
+    int rank = 0, start = 0;
+    for (int b = 0; b < 64; b++) {
+        const int other = __shfl(cnt, b);
+        const bool before = other > cnt || (other == cnt && b < L);
+        rank += before ? 1 : 0;
+        start += before ? other : 0;
+    }
+    order[rank] = L;
+    count_of[L] = cnt;
+    start_of[L] = start;
+    for (int i = 0, k = start; i < n; i++) {
+        const uint32_t w = natural[i];
+        if (bank_of(w) == L)
+            by_bank[k++] = w;
+    }
+    __syncthreads();
+    // the host's dealing, word by word (a24_pack.cpp: order_by_bank), on one lane
+    if (L == 0) {
+        const int rounds = (n + 63) / 64;
+        for (int r = 0; r < rounds; r++)
+            used[r] = 0;
+        for (int i = 0; i < 64; i++) {
+            const int b = order[i];
+            const int c = count_of[b];
+            if (c == 0)
+                break;
+            for (int r = 0; r < rounds; r++)
+                mine[r] = 0;
+            for (int j = 0; j < c; j++) {
+                int best = -1, best_free = 0;
+                for (int r = 0; r < rounds; r++) {
+                    const int free = (r == rounds - 1 ? n - 64 * (rounds - 1) : 64) - used[r];
+                    if (free > 0 && (best < 0 || mine[r] < mine[best] || (mine[r] == mine[best] && free > best_free))) {
+                        best = r;
+                        best_free = free;
+                    }
+                }
+                natural[best * 64 + used[best]++] = by_bank[start_of[b] + j];
+                mine[best]++;
+            }
+        }
+    }
+    __syncthreads();
+    for (int i = L; i < n; i += 64)
+        words[(size_t)begin + i] = natural[i];
+}
+
+}  // namespace
+
+// A2: row-major M x K fp16 in device memory (M % 128 == 0, K % 128 == 0, checked by the caller).
+// offsets: (M / 16) * (K / 128) + 1 ints; *longest: the longest list's length.
+extern "C" int a24_launch_residual_offsets(void* stream, const void* A2, int M, int K, int* offsets, int* longest)
+{
+    const int units = K / 128;
+    const long lists = static_cast<long>(M / 16) * units;
+    if (lists < 1 || lists > 0x7ffffff0L)
+        return static_cast<int>(hipErrorInvalidValue);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(a24_residual_count_kernel, dim3((unsigned)((lists + 3) / 4)), dim3(256), 0, s,
+                       static_cast<const uint16_t*>(A2), K, units, lists, offsets);
+    hipLaunchKernelGGL(a24_residual_scan_kernel, dim3(1), dim3(1024), 0, s, offsets, lists, longest);
+    return static_cast<int>(hipGetLastError());
+}
+
+// words: offsets[last] + 64 of them (the last 64 are zeroed).
+extern "C" int a24_launch_residual_words(void* stream, const void* A2, int M, int K, const int* offsets, void* words)
+{
+    const int units = K / 128;
+    const long lists = static_cast<long>(M / 16) * units;
+    if (lists < 1 || lists > 0x7ffffff0L)
+        return static_cast<int>(hipErrorInvalidValue);
+    hipLaunchKernelGGL(a24_residual_emit_kernel, dim3((unsigned)lists), dim3(64), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint16_t*>(A2), K, units, lists, offsets, static_cast<uint32_t*>(words));
+    return static_cast<int>(hipGetLastError());
+}
+
 // A second stream per caller stream, so that the residual's Tiled-CSL kernel can run beside the 2:4
 // kernel (the reference gives them two streams as well, kernel_benchmark/spmm_test.cu:459-461).
 // Default priority, created on first use, kept until the process ends; at most 32 caller

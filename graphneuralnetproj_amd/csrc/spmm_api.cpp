@@ -25,6 +25,8 @@ int a24_launch_spmm(void* stream, const void* packed, const void* B, void* out, 
                     int waves, int share_b, long ldb, long ldo, long slab, int residual_loads = 0,
                     const void* words = nullptr, const void* offsets = nullptr);
 int a24_launch_split_pack(void* stream, const void* A, void* packed, void* residual, int M, int K);
+int a24_launch_residual_offsets(void* stream, const void* A2, int M, int K, int* offsets, int* longest);
+int a24_launch_residual_words(void* stream, const void* A2, int M, int K, const int* offsets, void* words);
 int a24_side_begin(void* stream, void** side);
 int a24_side_end(void* stream, void* side);
 int tcsl_static_workspace(void** slabs, long* bytes);
@@ -647,6 +649,26 @@ extern "C" int HeteroSparse_SpMM_API(void* stream, const void* Packed_A1, const 
 extern "C" int HeteroSparse_PackA2(const uint16_t* A2_h, int M, int K, uint32_t** Words, int** Offsets, int* LongestList)
 {
     return a24::pack_residual(A2_h, M, K, Words, Offsets, LongestList);
+}
+
+extern "C" int HeteroSparse_DevicePackA2_Offsets(void* stream, const void* A2_d, int M, int K, int* Offsets_d, int* LongestList_d)
+{
+    if (!A2_d || !Offsets_d || !LongestList_d || M <= 0 || K <= 0 || M % (a24::kRows * a24::kGroupBlocks) != 0
+        || K % a24::kUnitCols != 0) {
+        std::fprintf(stderr, "HeteroSparse_DevicePackA2_Offsets: need M %% 128 == 0, K %% 128 == 0 and non-null pointers (M=%d K=%d)\n", M, K);
+        return tcsl_error_invalid_value();
+    }
+    return a24_launch_residual_offsets(stream, A2_d, M, K, Offsets_d, LongestList_d);
+}
+
+extern "C" int HeteroSparse_DevicePackA2_Words(void* stream, const void* A2_d, int M, int K, const int* Offsets_d, void* Words_d)
+{
+    if (!A2_d || !Offsets_d || !Words_d || M <= 0 || K <= 0 || M % (a24::kRows * a24::kGroupBlocks) != 0
+        || K % a24::kUnitCols != 0) {
+        std::fprintf(stderr, "HeteroSparse_DevicePackA2_Words: need M %% 128 == 0, K %% 128 == 0 and non-null pointers (M=%d K=%d)\n", M, K);
+        return tcsl_error_invalid_value();
+    }
+    return a24_launch_residual_words(stream, A2_d, M, K, Offsets_d, Words_d);
 }
 
 extern "C" int HeteroSparse_Fused_SpMM_API(void* stream, const void* Packed_A1, const void* A2_Words, const int* A2_Offsets,

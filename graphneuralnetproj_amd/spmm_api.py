@@ -60,6 +60,8 @@ EXPORTED_SYMBOLS = (
     "HeteroSparse_A1_Partials",
     "HeteroSparse_DeviceSplitPack",
     "HeteroSparse_PackA2",
+    "HeteroSparse_DevicePackA2_Offsets",
+    "HeteroSparse_DevicePackA2_Words",
     "HeteroSparse_Fused_SpMM_API",
 )
 
@@ -175,6 +177,12 @@ def load_library():
     lib.HeteroSparse_PackA2.restype = ctypes.c_int
     lib.HeteroSparse_PackA2.argtypes = [_u16p, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.POINTER(ctypes.c_uint32)),
                                         ctypes.POINTER(ctypes.POINTER(ctypes.c_int)), ctypes.POINTER(ctypes.c_int)]
+    lib.HeteroSparse_DevicePackA2_Offsets.restype = ctypes.c_int
+    lib.HeteroSparse_DevicePackA2_Offsets.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                                      ctypes.c_void_p]
+    lib.HeteroSparse_DevicePackA2_Words.restype = ctypes.c_int
+    lib.HeteroSparse_DevicePackA2_Words.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                                    ctypes.c_void_p]
     lib.HeteroSparse_Fused_SpMM_API.restype = ctypes.c_int
     lib.HeteroSparse_Fused_SpMM_API.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] + [ctypes.c_void_p] * 2 + [ctypes.c_int] * 3 + [
         ctypes.c_void_p, ctypes.c_int]
@@ -511,3 +519,32 @@ def split_pack_on_device(A_d, want_residual=True, stream=None):
     if rc != 0:
         raise SpMMError("HeteroSparse_DeviceSplitPack", rc, lib.SpMM_GetErrorString(rc).decode())
     return packed, residual
+
+
+def pack_residual_on_device(A2_d, stream=None):
+    """Residual lists (words int32 tensor of T + 64, offsets int32 tensor, longest list) of a torch CUDA
+    fp16 matrix, made on the GPU; same bits as HeteroSparse_PackA2.  Synchronises once, to size the words."""
+    import torch
+
+    lib = load_library()
+    M, K = A2_d.shape
+    if A2_d.dtype != torch.float16 or not A2_d.is_contiguous():
+        raise TypeError("expected a contiguous float16 CUDA tensor")
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    sp = ctypes.c_void_p(stream.cuda_stream) if stream.cuda_stream else None
+    lists = (M // 16) * (K // 128)
+    offsets = torch.empty(max(lists, 0) + 2, dtype=torch.int32, device=A2_d.device)  # the last int: the longest list
+    rc = lib.HeteroSparse_DevicePackA2_Offsets(sp, _ptr(A2_d), M, K, _ptr(offsets), ctypes.c_void_p(offsets.data_ptr() + 4 * (lists + 1)))
+    if rc != 0:
+        raise SpMMError("HeteroSparse_DevicePackA2_Offsets", rc, lib.SpMM_GetErrorString(rc).decode())
+    stream.synchronize()
+    total, longest = (int(x) for x in offsets[lists:lists + 2].cpu())
+    if total < 0:
+        raise SpMMError("HeteroSparse_DevicePackA2_Offsets", -1, "more residual values than an int counts")
+    words = torch.empty(total + 64, dtype=torch.int32, device=A2_d.device)
+    rc = lib.HeteroSparse_DevicePackA2_Words(sp, _ptr(A2_d), M, K, _ptr(offsets), _ptr(words))
+    if rc != 0:
+        raise SpMMError("HeteroSparse_DevicePackA2_Words", rc, lib.SpMM_GetErrorString(rc).decode())
+    return words, offsets[:lists + 1], longest
+

@@ -382,6 +382,24 @@ SPMM_EXPORT int HeteroSparse_A1_Partials(void* stream, const void* Packed_A1, co
  * hipError_t value: hipErrorUnknown for N outside {8, 16, 32, 64}; hipErrorInvalidValue for M % 128,
  * K % 128, an empty batch, a list too long, a missing pointer.  Only enqueues work on `stream`.
  */
+/*
+ * HeteroSparse_PackA2 on the GPU, for a residual that is already in device memory (the A2_d that
+ * HeteroSparse_DeviceSplitPack wrote): the same words in the same order.  Two steps, because the
+ * caller owns the buffers and their size depends on the data:
+ *   HeteroSparse_DevicePackA2_Offsets  fills Offsets_d ((M/16)*(K/128) + 1 ints; the last one, T, is
+ *                                      the number of words, -1 if it would not fit an int) and
+ *                                      *LongestList_d (one int);
+ *   HeteroSparse_DevicePackA2_Words    fills Words_d (T + 64 words, the last 64 zero) from A2_d and
+ *                                      those offsets.
+ * Both only enqueue kernels on `stream`; read T and the longest list back (after synchronising) to
+ * size the second buffer, or allocate the worst case M*K/2 + 64 words up front.  Return a hipError_t
+ * value; hipErrorInvalidValue for M % 128, K % 128 or null pointers.
+ */
+SPMM_EXPORT int HeteroSparse_DevicePackA2_Offsets(void* stream, const void* A2_d, int M_Global, int K_Global, int* Offsets_d,
+                                                  int* LongestList_d);
+SPMM_EXPORT int HeteroSparse_DevicePackA2_Words(void* stream, const void* A2_d, int M_Global, int K_Global,
+                                                const int* Offsets_d, void* Words_d);
+
 #define HETERO_FUSED_MAX_LIST 320
 SPMM_EXPORT int HeteroSparse_PackA2(const uint16_t* A2_h, int M_Global, int K_Global, uint32_t** Words, int** Offsets,
                                     int* LongestList);

@@ -501,3 +501,39 @@ def test_fused_hip_graph_replays_match_eager(spmm, oracle):
         torch.cuda.synchronize()
         assert torch.equal(d_C, want)
 
+
+@pytest.mark.parametrize("M,K,sparsity,skew", [(128, 128, 0.5, False), (256, 640, 0.45, False), (1024, 2048, 0.7, False),
+                                               (128, 128, 1.0, False), (384, 256, 0.0, False), (512, 512, 0.5, True),
+                                               (256, 128, 0.97, False)])
+def test_device_residual_lists_equal_host(spmm, oracle, M, K, sparsity, skew):
+    """The GPU's residual lists against the host's, bit for bit (words, offsets, longest list, the 64
+    words of padding), with -0, NaN, denormal and infinity patterns, lists of one round (left as
+    collected), of several (ordered by bank) and of the maximum length (a dense matrix: 1024)."""
+    torch = _torch()
+    A = spmm.synth_weights(M, K, sparsity, skew, seed=M + K + 7)
+    A.view(np.uint16)[0, :8] = [0x8000, 0x7E00, 0x0001, 0x3C00, 0xFC00, 0x8001, 0, 0x7C00]
+    A.view(np.uint16)[17, 4:8] = [0x7E00, 0x8000, 0xFE00, 0x0001]
+    _, A2 = oracle.decompose(A)
+    want_words, want_offs, want_longest = spmm.HeteroSparse_PackA2(A2)
+    d_A2 = torch.from_numpy(A2.view(np.int16).copy()).to("cuda:0").view(torch.float16)
+    print(f"[gpu case] device residual lists M={M} K={K} sparsity={sparsity} skew={skew}", flush=True)
+    words, offs, longest = spmm.pack_residual_on_device(d_A2)
+    torch.cuda.synchronize()
+    assert longest == want_longest
+    assert np.array_equal(offs.cpu().numpy(), want_offs)
+    assert np.array_equal(words.cpu().numpy().view(np.uint32), want_words)
+    # and from the GPU's own split, through the one-launch product
+    d_A = torch.from_numpy(A.view(np.int16).copy()).to("cuda:0").view(torch.float16)
+    packed, residual = spmm.split_pack_on_device(d_A)
+    words2, offs2, longest2 = spmm.pack_residual_on_device(residual)
+    assert torch.equal(words2, words) and torch.equal(offs2, offs) and longest2 == longest
+    if longest <= spmm.HETERO_FUSED_MAX_LIST:
+        N = 16
+        Bh = spmm.synth_activations(N, K, seed=3)
+        d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device="cuda:0")
+        spmm.HeteroSparse_Fused_SpMM_API(torch.cuda.current_stream(), packed, words2, offs2, longest2, _dev(Bh), d_C, M, N, K,
+                                         None, 1)
+        torch.cuda.synchronize()
+        rows = np.isfinite(A).all(axis=1)  # the product is NaN in the rows that hold NaN or infinity: compare the others
+        assert_close(d_C.cpu().numpy()[:, rows], oracle.gemm_f32(np.ascontiguousarray(A[rows]), Bh))
+
