@@ -213,6 +213,9 @@ def sweep(G, lib, torch, dev, sptr, with_stack):
         out.append(split_case(G, lib, torch, dev, sptr, "opt30b_ffn1", 16, sparsity))
     if with_stack:
         out.append(stack_step(G, torch, dev))
+        # the same stack at a sparsity where the fork's split pays, in both forms
+        out.append(stack_step(G, torch, dev, sparsity=0.6))
+        out.append(stack_step(G, torch, dev, sparsity=0.6, split=True))
     return out
 
 
@@ -284,14 +287,16 @@ def split_case(G, lib, torch, dev, sptr, workload, N, sparsity):
             "ms": best, "frac": one_bytes / (best * 1e-3) / 1e9 / HBM_PEAK_GBPS}
 
 
-def stack_step(G, torch, dev, layers=64, h=9216, N=16, sparsity=0.8):
+def stack_step(G, torch, dev, layers=64, h=9216, N=16, sparsity=0.8, split=False):
     """64 OPT-66B-shaped blocks, random-init weights drawn and encoded on the GPU (about 52 GB
-    resident): time per token step, eager and as a HIP graph."""
+    resident at 80 % sparsity): time per token step, eager and as a HIP graph.  split: every weight
+    as 2:4 records + residual lists, one launch per product, instead of Tiled-CSL."""
     from graphneuralnetproj_amd import decoder_stack as DS
 
     torch.cuda.empty_cache()
     t0 = time.perf_counter()
-    blocks = [DS.build_layer_on_device(G, torch, dev, h, N, sparsity, seed=1 + i)[0] for i in range(layers)]
+    build = DS.build_split_layer_on_device if split else DS.build_layer_on_device
+    blocks = [build(G, torch, dev, h, N, sparsity, seed=1 + i)[0] for i in range(layers)]
     torch.cuda.synchronize()
     build_s = time.perf_counter() - t0
     stack = DS.Stack(G, torch, blocks, h, N)
@@ -310,6 +315,7 @@ def stack_step(G, torch, dev, layers=64, h=9216, N=16, sparsity=0.8):
         times.append((time.perf_counter() - t0) * 1e3 / 5)
     eager_ms = float(np.median(times))
     graph_ms = None
+    g = None
     try:
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
@@ -329,7 +335,11 @@ def stack_step(G, torch, dev, layers=64, h=9216, N=16, sparsity=0.8):
         print(f"bench.py: graph capture of the stack failed: {e}", file=sys.stderr)
     weight_bytes = sum(L.bytes() for L in blocks)
     ms = min(eager_ms, graph_ms) if graph_ms else eager_ms
-    return {"case": "decoder_stack", "layers": layers, "hidden": h, "N": N, "sparsity": sparsity,
+    del stack, blocks, g
+    torch.cuda.empty_cache()
+    case = "decoder_stack" if sparsity == 0.8 and not split else f"decoder_stack_{int(sparsity * 100)}pct" + ("_split" if split else "")
+    return {"case": case, "layers": layers, "hidden": h, "N": N, "sparsity": sparsity,
+            "form": "2:4 records + residual lists, one launch per product" if split else "Tiled-CSL",
             "weights": "random-init per layer, drawn and encoded on the GPU", "resident_weight_bytes": weight_bytes,
             "ms": ms, "eager_ms": eager_ms, "graph_ms": graph_ms, "frac": weight_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "hbm_floor_ms": weight_bytes / (HBM_PEAK_GBPS * 1e9) * 1e3, "build_s": build_s}

@@ -251,7 +251,7 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
                                                                      _Float16* __restrict__ out, int units,
                                                                      int units_per_batch, long ldb, long ldo, long slab,
                                                                      int n_tokens, const unsigned* __restrict__ words,
-                                                                     const int* __restrict__ offsets)
+                                                                     const int* __restrict__ offsets, int relu)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char tile[];  // [2][NT * 16][kRowBytes], then [W][kImageBytes]
     constexpr int kBuf = NT * 16 * kRowBytes;
@@ -527,6 +527,8 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
                 float4v s = acc[r][t];
                 if constexpr (RL > 0)
                     s += accd[r][t];
+                if (relu)
+                    s = float4v{fmaxf(s[0], 0.f), fmaxf(s[1], 0.f), fmaxf(s[2], 0.f), fmaxf(s[3], 0.f)};
                 half4 h = {static_cast<_Float16>(s[0]), static_cast<_Float16>(s[1]), static_cast<_Float16>(s[2]),
                            static_cast<_Float16>(s[3])};
                 *reinterpret_cast<half4*>(dstc + (size_t)n * ldo + (block0 + r) * 16 + (lane >> 4) * 4) = h;
@@ -537,7 +539,7 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
 
 template<int NT, int RB, int W, int RL>
 int launch_shared_b(hipStream_t stream, const void* packed, const void* B, void* out, int M, int N, int K, int split_k,
-                    long ldb, long ldo, long slab, const void* words, const void* offsets)
+                    long ldb, long ldo, long slab, const void* words, const void* offsets, int relu)
 {
     const int units = K / 128;
     const int per_batch = (units + split_k - 1) / split_k;
@@ -552,7 +554,7 @@ int launch_shared_b(hipStream_t stream, const void* packed, const void* B, void*
     }
     hipLaunchKernelGGL(kern, dim3(M / (16 * RB * W), split_k), dim3(W * kWave), lds, stream,
                        static_cast<const uint8_t*>(packed), static_cast<const _Float16*>(B), static_cast<_Float16*>(out), units,
-                       per_batch, ldb, ldo, slab, N, static_cast<const unsigned*>(words), static_cast<const int*>(offsets));
+                       per_batch, ldb, ldo, slab, N, static_cast<const unsigned*>(words), static_cast<const int*>(offsets), relu);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -560,11 +562,11 @@ int launch_shared_b(hipStream_t stream, const void* packed, const void* B, void*
 // shapes only: two row blocks per wave, four or eight waves.
 template<int NT>
 int launch_shared_b_nt(hipStream_t s, const void* packed, const void* B, void* out, int M, int N, int K, int split_k, int rb,
-                       int waves, long ldb, long ldo, long slab, int rl, const void* words, const void* offsets)
+                       int waves, long ldb, long ldo, long slab, int rl, const void* words, const void* offsets, int relu)
 {
 #define A24_CASE(RB_, W_, RL_)                   \
     if (rb == RB_ && waves == W_ && rl == RL_) \
-        return launch_shared_b<NT, RB_, W_, RL_>(s, packed, B, out, M, N, K, split_k, ldb, ldo, slab, words, offsets);
+        return launch_shared_b<NT, RB_, W_, RL_>(s, packed, B, out, M, N, K, split_k, ldb, ldo, slab, words, offsets, relu);
     A24_CASE(2, 4, 0) A24_CASE(2, 8, 0)
     A24_CASE(2, 4, 1) A24_CASE(2, 8, 1) A24_CASE(2, 4, 2) A24_CASE(2, 8, 2) A24_CASE(2, 4, 3) A24_CASE(2, 8, 3)
     A24_CASE(2, 4, 4) A24_CASE(2, 4, 5)
@@ -615,22 +617,23 @@ int launch_nt(hipStream_t s, const void* packed, const void* B, void* out, int M
 // Batch b of ceil((K/128)/split_k) units writes fp16 [N][ldo] to out + b * slab.  The caller has
 // checked: M % (16 * rb) == 0 (share_b: M % (16 * rb * waves) == 0), K % 128 == 0, N in {8, 16, 32, 64}, no batch empty, pointers set.
 // residual_loads > 0 (share_b with rb == 2 only): the launch also multiplies the residual lists
-// words / offsets, none longer than 64 * residual_loads words.
+// words / offsets, none longer than 64 * residual_loads words.  relu (share_b only): negative
+// results are written as zero (for a launch that writes the finished result).
 extern "C" int a24_launch_spmm(void* stream, const void* packed, const void* B, void* out, int M, int N, int K,
                                int split_k, int rb, int waves, int share_b, long ldb, long ldo, long slab,
-                               int residual_loads, const void* words, const void* offsets)
+                               int residual_loads, const void* words, const void* offsets, int relu)
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (share_b) {  // waves own rows and share the activation tile through LDS
         switch (N) {
             case 8:
-            case 16: return launch_shared_b_nt<1>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets);
-            case 32: return launch_shared_b_nt<2>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets);
-            case 64: return launch_shared_b_nt<4>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets);
+            case 16: return launch_shared_b_nt<1>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets, relu);
+            case 32: return launch_shared_b_nt<2>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets, relu);
+            case 64: return launch_shared_b_nt<4>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets, relu);
             default: return static_cast<int>(hipErrorInvalidValue);
         }
     }
-    if (residual_loads != 0)
+    if (residual_loads != 0 || relu)
         return static_cast<int>(hipErrorInvalidValue);
     switch (N) {
         case 8:

@@ -23,7 +23,7 @@ int tcsl_launch_encode_offsets(void* stream, const void* A, int M, int K, int* o
 int tcsl_launch_encode_items(void* stream, const void* A, int M, int K, const int* offsets, void* items);
 int a24_launch_spmm(void* stream, const void* packed, const void* B, void* out, int M, int N, int K, int split_k, int rb,
                     int waves, int share_b, long ldb, long ldo, long slab, int residual_loads = 0,
-                    const void* words = nullptr, const void* offsets = nullptr);
+                    const void* words = nullptr, const void* offsets = nullptr, int relu = 0);
 int a24_launch_split_pack(void* stream, const void* A, void* packed, void* residual, int M, int K);
 int a24_launch_residual_offsets(void* stream, const void* A2, int M, int K, int* offsets, int* longest);
 int a24_launch_residual_words(void* stream, const void* A2, int M, int K, const int* offsets, void* words);
@@ -671,9 +671,10 @@ extern "C" int HeteroSparse_DevicePackA2_Words(void* stream, const void* A2_d, i
     return a24_launch_residual_words(stream, A2_d, M, K, Offsets_d, Words_d);
 }
 
-extern "C" int HeteroSparse_Fused_SpMM_API(void* stream, const void* Packed_A1, const void* A2_Words, const int* A2_Offsets,
-                                           int LongestList, const void* B, void* C, int M, int N, int K,
-                                           void* Reduction_Workspace, int Split_K)
+namespace {
+
+int fused_call(const char* who, void* stream, const void* Packed_A1, const void* A2_Words, const int* A2_Offsets, int LongestList,
+               const void* B, long ldb, void* C, long ldc, int M, int N, int K, void* Reduction_Workspace, int Split_K, int Flags)
 {
     if (N != 8 && N != 16 && N != 32 && N != 64) {
         std::printf("MM_Sparse_API Error: Unsupported N dimension %d!\n", N);  // csrc/SpMM_API.cu:192-193
@@ -683,16 +684,38 @@ extern "C" int HeteroSparse_Fused_SpMM_API(void* stream, const void* Packed_A1, 
     const int loads = (LongestList + 63) / 64;
     const int waves = (N == 64 && loads >= 4) ? 4 : a24_waves_for(M > 0 ? M : 128, Split_K);  // the former: what fits the registers
     if (!Packed_A1 || !A2_Words || !A2_Offsets || !B || !C || LongestList < 0 || LongestList > HETERO_FUSED_MAX_LIST
-        || !a24_shape_ok(M, N, K, Split_K, 2, waves, 1) || (Split_K > 1 && !Reduction_Workspace)) {
-        std::fprintf(stderr, "HeteroSparse_Fused_SpMM_API: unsupported call M=%d N=%d K=%d Split_K=%d LongestList=%d (need M %% 128 == 0, K %% 128 == 0, no empty batch, lists of at most %d words, non-null pointers)\n",
-                     M, N, K, Split_K, LongestList, HETERO_FUSED_MAX_LIST);
+        || !a24_shape_ok(M, N, K, Split_K, 2, waves, 1) || (Split_K > 1 && !Reduction_Workspace) || ldb < K || ldc < M
+        || ldb % 8 != 0 || ldc % 8 != 0 || (Flags & ~SPMM_FLAG_RELU)) {
+        std::fprintf(stderr, "%s: unsupported call M=%d N=%d K=%d Split_K=%d LongestList=%d ldb=%ld ldc=%ld (need M %% 128 == 0, K %% 128 == 0, no empty batch, lists of at most %d words, strides that are multiples of 8 and hold a vector, non-null pointers)\n",
+                     who, M, N, K, Split_K, LongestList, ldb, ldc, HETERO_FUSED_MAX_LIST);
         return tcsl_error_invalid_value();
     }
+    const int relu = (Flags & SPMM_FLAG_RELU) ? 1 : 0;
     const long mn = static_cast<long>(M) * N;
-    void* out = Split_K == 1 ? C : Reduction_Workspace;
-    const int rc = a24_launch_spmm(stream, Packed_A1, B, out, M, N, K, Split_K, 2, waves, 1, K, M, mn, loads, A2_Words,
-                                   A2_Offsets);
-    if (rc != 0 || Split_K == 1)
+    if (Split_K == 1)
+        return a24_launch_spmm(stream, Packed_A1, B, C, M, N, K, 1, 2, waves, 1, ldb, ldc, mn, loads, A2_Words, A2_Offsets, relu);
+    const int rc = a24_launch_spmm(stream, Packed_A1, B, Reduction_Workspace, M, N, K, Split_K, 2, waves, 1, ldb, M, mn, loads,
+                                   A2_Words, A2_Offsets, 0);
+    if (rc != 0)
         return rc;
-    return tcsl_launch_reduce(stream, C, static_cast<uint16_t*>(Reduction_Workspace), mn, 1, mn, Split_K, 0);
+    return tcsl_launch_reduce(stream, C, static_cast<uint16_t*>(Reduction_Workspace), M, N, ldc, Split_K, relu);
+}
+
+}  // namespace
+
+extern "C" int HeteroSparse_Fused_SpMM_API(void* stream, const void* Packed_A1, const void* A2_Words, const int* A2_Offsets,
+                                           int LongestList, const void* B, void* C, int M, int N, int K,
+                                           void* Reduction_Workspace, int Split_K)
+{
+    return fused_call("HeteroSparse_Fused_SpMM_API", stream, Packed_A1, A2_Words, A2_Offsets, LongestList, B, K, C, M, M, N, K,
+                      Reduction_Workspace, Split_K, 0);
+}
+
+extern "C" int HeteroSparse_Fused_SpMM_API_Strided(void* stream, const void* Packed_A1, const void* A2_Words,
+                                                   const int* A2_Offsets, int LongestList, const void* B, long ldb, void* C,
+                                                   long ldc, int M, int N, int K, void* Reduction_Workspace, int Split_K,
+                                                   int Flags)
+{
+    return fused_call("HeteroSparse_Fused_SpMM_API_Strided", stream, Packed_A1, A2_Words, A2_Offsets, LongestList, B, ldb, C, ldc,
+                      M, N, K, Reduction_Workspace, Split_K, Flags);
 }

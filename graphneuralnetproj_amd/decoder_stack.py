@@ -35,12 +35,23 @@ class Layer:
     def __init__(self, mats):
         self.mats = mats
 
+    @staticmethod
+    def is_split(mat):
+        return isinstance(mat[0], tuple)
+
     def clone(self):
         return Layer({k: (it.clone() if it is not None else None, of if it is not None else of.clone(), M, K, s)
                       for k, (it, of, M, K, s) in self.mats.items()})
 
     def bytes(self):
-        return sum((it.numel() * 4 if it is not None else of.numel() * 2) for it, of, _, _, _ in self.mats.values())
+        total = 0
+        for mat in self.mats.values():
+            it, of = mat[0], mat[1]
+            if Layer.is_split(mat):  # ((records, words), (list offsets, longest list), M, K, split_k)
+                total += it[0].numel() + 4 * (it[1].numel() - 64)
+            else:
+                total += it.numel() * 4 if it is not None else of.numel() * 2
+        return total
 
 
 def layer_shapes(h):
@@ -88,10 +99,36 @@ def build_layer_on_device(G, torch, dev, h, N, sparsity, seed, weight_std=0.02, 
     return Layer(mats), samples
 
 
+def build_split_layer_on_device(G, torch, dev, h, N, sparsity, seed, weight_std=0.02, sample_rows=0):
+    """build_layer_on_device with every weight split into a 2:4 part (records for the sparse matrix
+    instruction) and a residual (lists), the fork's decomposition (kernel_benchmark/spmm_decompose.h:12-51),
+    for the one-launch product.  Same random matrices as build_layer_on_device gives for the seed.
+    A matrix is ((records, words), (list offsets, longest list), M, K, split_k)."""
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    mats, samples = {}, {}
+    for name, (M, K) in layer_shapes(h).items():
+        A = torch.randn((M, K), generator=gen, device=dev, dtype=torch.float32)
+        A.mul_(weight_std)
+        A.mul_(torch.rand((M, K), generator=gen, device=dev) >= sparsity)
+        A = A.to(torch.float16)
+        records, residual = G.split_pack_on_device(A)
+        words, offsets, longest = G.pack_residual_on_device(residual)
+        if longest > G.HETERO_FUSED_MAX_LIST:
+            raise ValueError(f"{name}: a residual list of {longest} words; the one-launch product takes {G.HETERO_FUSED_MAX_LIST}")
+        mats[name] = ((records, words), (offsets, longest), M, K, G.HeteroSparse_SuggestSplitK(M, N, K))
+        if sample_rows:
+            rows = torch.randperm(M, generator=gen, device=dev)[:sample_rows].sort().values
+            samples[name] = (rows.cpu().numpy(), A[rows].cpu().numpy())
+        del A, residual
+    return Layer(mats), samples
+
+
 class Stack:
     def __init__(self, G, torch, layers, h, N):
         self.G, self.torch, self.layers, self.h, self.N = G, torch, layers, h, N
-        dev = layers[0].mats["qkv"][1].device
+        first = layers[0].mats["qkv"]
+        dev = (first[1][0] if Layer.is_split(first) else first[1]).device
         f16 = torch.float16
         self.x = [torch.zeros((N, h), dtype=f16, device=dev) for _ in range(2)]  # ping-pong layer inputs
         self.qkv = torch.zeros((N, 3 * h), dtype=f16, device=dev)
@@ -103,7 +140,10 @@ class Stack:
 
     def _product(self, stream, mat, src, ldb, dst, ldc, flags=0):
         it, of, M, K, s = mat
-        if it is not None:
+        if Layer.is_split(mat):
+            self.G.HeteroSparse_Fused_SpMM_API_Strided(stream, it[0], it[1], of[0], of[1], src, ldb, dst, ldc, M, self.N, K,
+                                                       self.ws, s, flags)
+        elif it is not None:
             self.G.SpMM_SplitK_API_Strided(stream, it, of, src, ldb, dst, ldc, M, self.N, K, self.ws, s, flags)
         else:  # dense on disk: [N][K] x [K][M] on the library GEMM (torch's current stream)
             self.torch.mm(src[:, :K], of, out=dst[:, :M])
@@ -137,6 +177,9 @@ def main():
                     help="device: every layer's weights are drawn and encoded on the GPU (default); host: drawn and "
                          "encoded on the host by the library's generator and encoder; copied: one host-made layer, "
                          "copied in HBM for the others")
+    ap.add_argument("--split", action="store_true",
+                    help="split every weight into a 2:4 part and a residual and multiply both in one launch "
+                         "(worth it up to about 70 %% sparsity); weights are made on the GPU")
     ap.add_argument("--model-dir", help="run rank 0 of a converted one-rank model directory (<dir>/1-gpu/, written by "
                                         "graphneuralnetproj_amd.model_files) instead of synthetic weights")
     args = ap.parse_args()
@@ -158,7 +201,9 @@ def main():
         args.layers, h = model_files.read_config(rank_dir)
         layers = model_files.upload_layers(model_files.load_rank(rank_dir, 0, 1), dev, tokens=N)
     else:
-        if args.weights == "device":
+        if args.split:
+            layers = [build_split_layer_on_device(G, torch, dev, h, N, args.sparsity, seed=1 + i)[0] for i in range(args.layers)]
+        elif args.weights == "device":
             layers = [build_layer_on_device(G, torch, dev, h, N, args.sparsity, seed=1 + i)[0] for i in range(args.layers)]
         else:
             first, _ = build_layer(G, torch, dev, h, N, args.sparsity, seed=1)
@@ -220,6 +265,7 @@ def main():
         "eager_ms": eager_ms, "graph_ms": graph_ms, "graph_matches_eager": graph_matches,
         "config": {"workload": f"{args.layers} layers x (QKV, out-proj, FFN1+ReLU, FFN2), h={h}, N={N}, "
                                f"{args.sparsity * 100:.0f}% sparse",
+                   "form": "2:4 records + residual lists, one launch per product" if args.split else "Tiled-CSL",
                    "weights": "model directory" if args.model_dir else
                    {"device": "random-init per layer, drawn and encoded on the GPU",
                     "host": "random-init per layer, drawn and encoded on the host",

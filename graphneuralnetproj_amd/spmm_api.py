@@ -63,6 +63,7 @@ EXPORTED_SYMBOLS = (
     "HeteroSparse_DevicePackA2_Offsets",
     "HeteroSparse_DevicePackA2_Words",
     "HeteroSparse_Fused_SpMM_API",
+    "HeteroSparse_Fused_SpMM_API_Strided",
 )
 
 
@@ -186,6 +187,10 @@ def load_library():
     lib.HeteroSparse_Fused_SpMM_API.restype = ctypes.c_int
     lib.HeteroSparse_Fused_SpMM_API.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] + [ctypes.c_void_p] * 2 + [ctypes.c_int] * 3 + [
         ctypes.c_void_p, ctypes.c_int]
+    lib.HeteroSparse_Fused_SpMM_API_Strided.restype = ctypes.c_int
+    lib.HeteroSparse_Fused_SpMM_API_Strided.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int, ctypes.c_void_p, ctypes.c_long,
+                                                        ctypes.c_void_p, ctypes.c_long] + [ctypes.c_int] * 3 + [
+        ctypes.c_void_p, ctypes.c_int, ctypes.c_int]
     lib.HeteroSparse_A1_Partials.restype = ctypes.c_int
     lib.HeteroSparse_A1_Partials.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 7
     _lib = lib
@@ -482,6 +487,20 @@ def HeteroSparse_Fused_SpMM_API(stream, Packed_A1, A2_Words, A2_Offsets, Longest
                                          _ptr(Reduction_Workspace), Split_K)
     if rc != 0:
         raise SpMMError("HeteroSparse_Fused_SpMM_API", rc, lib.SpMM_GetErrorString(rc).decode())
+    return rc
+
+
+def HeteroSparse_Fused_SpMM_API_Strided(stream, Packed_A1, A2_Words, A2_Offsets, LongestList, B, ldb, C, ldc, M_Global, N_Global,
+                                        K_Global, Reduction_Workspace, Split_K, Flags=0):
+    """HeteroSparse_Fused_SpMM_API with token strides ldb / ldc (elements) and Flags (SPMM_FLAG_RELU)."""
+    lib = load_library()
+    if stream is not None and not isinstance(stream, int):
+        stream = stream.cuda_stream
+    rc = lib.HeteroSparse_Fused_SpMM_API_Strided(ctypes.c_void_p(stream) if stream else None, _ptr(Packed_A1), _ptr(A2_Words),
+                                                 _ptr(A2_Offsets), LongestList, _ptr(B), ldb, _ptr(C), ldc, M_Global, N_Global,
+                                                 K_Global, _ptr(Reduction_Workspace), Split_K, Flags)
+    if rc != 0:
+        raise SpMMError("HeteroSparse_Fused_SpMM_API_Strided", rc, lib.SpMM_GetErrorString(rc).decode())
     return rc
 
 

@@ -407,6 +407,16 @@ SPMM_EXPORT int HeteroSparse_Fused_SpMM_API(void* stream, const void* Packed_A1,
                                             int LongestList, const void* B, void* C, int M_Global, int N_Global,
                                             int K_Global, void* Reduction_Workspace, int Split_K);
 
+/*
+ * HeteroSparse_Fused_SpMM_API for activations and results inside wider per-token buffers
+ * (B[n*ldb + k], C[n*ldc + m], ldb >= K, ldc >= M, multiples of 8 elements) with an optional clamp
+ * (Flags = 0 or SPMM_FLAG_RELU), like SpMM_SplitK_API_Strided: what a chain of decoder layers needs.
+ */
+SPMM_EXPORT int HeteroSparse_Fused_SpMM_API_Strided(void* stream, const void* Packed_A1, const void* A2_Words,
+                                                    const int* A2_Offsets, int LongestList, const void* B, long ldb, void* C,
+                                                    long ldc, int M_Global, int N_Global, int K_Global,
+                                                    void* Reduction_Workspace, int Split_K, int Flags);
+
 #ifdef __cplusplus
 }
 #endif
