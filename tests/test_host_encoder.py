@@ -24,6 +24,15 @@ def test_library_exports_every_declared_symbol(spmm):
     assert sorted(declared) == sorted(spmm_api.EXPORTED_SYMBOLS)
 
 
+def test_mirror_constants_equal_the_headers(spmm):
+    """The flag and limit values of the Python mirror are the header's."""
+    header = open(os.path.join(ROOT, "include", "SpMM_API.h")).read()
+    defines = {name: int(value) for name, value in re.findall(r"#define\s+((?:SPMM_FLAG|HETERO)_\w+)\s+(\d+)", header)}
+    assert len(defines) >= 5
+    for name, value in defines.items():
+        assert getattr(spmm, name) == value, name
+
+
 def test_product_encoder_matches_golden_small(spmm):
     z = np.load(os.path.join(GOLD, "encoder_small.npz"))
     names = sorted({k.rsplit(".", 1)[0] for k in z.files})
