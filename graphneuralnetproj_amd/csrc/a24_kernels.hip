@@ -280,12 +280,14 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
         src[i] = B + (size_t)n * ldb + (c & 15) * 8;
         dst[i] = n * kRowBytes + (c & 15) * 16;
     }
-    // where this lane's fragments sit in a buffer
+    // where this lane's fragments sit in a buffer (with more than 16 tokens every token block is
+    // full, so the blocks are a constant apart: one register instead of NT)
     int frag[NT];
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         int n = t * 16 + (lane & 15);
-        n = n < n_tokens ? n : n_tokens - 1;
+        if (NT == 1)
+            n = n < n_tokens ? n : n_tokens - 1;
         frag[t] = n * kRowBytes + (lane >> 4) * 16;
     }
 
@@ -569,9 +571,9 @@ int launch_shared_b_nt(hipStream_t s, const void* packed, const void* B, void* o
         return launch_shared_b<NT, RB_, W_, RL_>(s, packed, B, out, M, N, K, split_k, ldb, ldo, slab, words, offsets, relu);
     A24_CASE(2, 4, 0) A24_CASE(2, 8, 0)
     A24_CASE(2, 4, 1) A24_CASE(2, 8, 1) A24_CASE(2, 4, 2) A24_CASE(2, 8, 2) A24_CASE(2, 4, 3) A24_CASE(2, 8, 3)
-    A24_CASE(2, 4, 4) A24_CASE(2, 4, 5)
+    A24_CASE(2, 4, 4) A24_CASE(2, 4, 5) A24_CASE(2, 8, 4)
     if constexpr (NT <= 2) {
-        A24_CASE(2, 8, 4) A24_CASE(2, 8, 5)  // with 64 tokens they would not fit 256 registers  // three record sets of four row blocks do not fit the registers beside 64 tokens
+        A24_CASE(2, 8, 5)  // with 64 tokens it would not fit 256 registers  // three record sets of four row blocks do not fit the registers beside 64 tokens
         A24_CASE(4, 2, 0) A24_CASE(4, 4, 0) A24_CASE(4, 8, 0)
     }
 #undef A24_CASE

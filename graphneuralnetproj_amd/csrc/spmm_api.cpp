@@ -682,7 +682,7 @@ int fused_call(const char* who, void* stream, const void* Packed_A1, const void*
     }
     // two row blocks per wave, activation tile shared through LDS: the one layout that takes the residual along
     const int loads = (LongestList + 63) / 64;
-    const int waves = (N == 64 && loads >= 4) ? 4 : a24_waves_for(M > 0 ? M : 128, Split_K);  // the former: what fits the registers
+    const int waves = (N == 64 && loads >= 5) ? 4 : a24_waves_for(M > 0 ? M : 128, Split_K);  // the former: what fits the registers
     if (!Packed_A1 || !A2_Words || !A2_Offsets || !B || !C || LongestList < 0 || LongestList > HETERO_FUSED_MAX_LIST
         || !a24_shape_ok(M, N, K, Split_K, 2, waves, 1) || (Split_K > 1 && !Reduction_Workspace) || ldb < K || ldc < M
         || ldb % 8 != 0 || ldc % 8 != 0 || (Flags & ~SPMM_FLAG_RELU)) {
