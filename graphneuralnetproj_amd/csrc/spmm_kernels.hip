@@ -168,13 +168,6 @@ __device__ __forceinline__ void store_through(_Float16* p, half4 v)
     __hip_atomic_store(reinterpret_cast<uint64_t*>(p), __builtin_bit_cast(uint64_t, v), __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_SYSTEM);
 }
-__device__ __forceinline__ void store_through(_Float16* p, half8 v)
-{
-    typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
-    const u64x2 w = __builtin_bit_cast(u64x2, v);
-    __hip_atomic_store(reinterpret_cast<uint64_t*>(p), w[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    __hip_atomic_store(reinterpret_cast<uint64_t*>(p) + 1, w[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-}
 __device__ __forceinline__ half8 load_through(const _Float16* p)
 {
     typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
@@ -295,10 +288,11 @@ __device__ __forceinline__ void fused_reduction_tail(const _Float16* __restrict_
 
 // ldb = elements between two tokens' vectors in B, ldo = the same for the output (column-major
 // only; the slabs of partial sums use M); relu != 0 clamps the output at zero (final results only).
-// arrivals != nullptr (Split_K > 1, column-major): `out` receives the slabs of partial sums as usual,
-// and the last workgroup to finish a group of rows adds the slabs up into fused_out (token stride
-// ldc, clamped if relu) itself; arrivals are counted in arrivals[blockIdx.x] (device memory, zero
-// before the launch and after it).
+// arrivals != nullptr (KSPLIT, Split_K > 1, column-major): `out` receives the slabs of partial sums
+// as usual, and the last workgroup to finish a tile row adds the slabs up into fused_out (token
+// stride ldc, clamped if relu) itself; arrivals are counted in arrivals[blockIdx.x] (device memory,
+// zero before the launch and after it).  The row-sharing layout always leaves the sum to the
+// reduction kernel (one workgroup would be left with W x 128 rows of every slab: measured slower).
 // blockDim.x = W * 64, grid = (groups of tile rows, Split_K).  Wave w of workgroup (g, b) owns
 // tile row g * W + w of batch b; with KSPLIT the workgroup owns tile row g and its waves share
 // the batch.  avg = tiles per batch = ceil((K / 64) / Split_K).  NB = number of 16-token column blocks;
@@ -454,9 +448,9 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         clear_tile(tile, lane);
     if (BLDS)
         __syncthreads();  // the only barrier: every wave of the workgroup reaches it
-    if (!KSPLIT && !active && !arrivals && BSW == 0)
-        return;  // (with the fused reduction every wave has to reach the barriers at the end)
-    const bool clamp = relu && !arrivals;  // partial sums are never clamped
+    if (!KSPLIT && !active && BSW == 0)
+        return;
+    const bool clamp = relu && !(KSPLIT && arrivals);  // partial sums are never clamped
 
     auto tile_range = [&](int i, int& begin, int& end) __attribute__((always_inline)) {  // 0 <= i < ntile
         if (i + 1 - wbase >= kWave) {  // slide the window (more than 63 tiles per wave only)
@@ -905,23 +899,16 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
             const int e = i * kWave + lane;
             const int tok = e >> 4, part = e & 15;
             const half8 v = *reinterpret_cast<const half8*>(tile + tok * kTokStride + part * 16);
-            _Float16* dst = oslab + (size_t)(c * 16 + tok) * ldo + part * 8;
-            if (arrivals)
-                store_through(dst, v);
-            else
-                *reinterpret_cast<half8*>(dst) = v;
+            *reinterpret_cast<half8*>(oslab + (size_t)(c * 16 + tok) * ldo + part * 8) = v;
         }
     }
     };
     if (KSPLIT || active)
         write_out();
-    if (ROWMAJ || !arrivals)
+    if (!KSPLIT || ROWMAJ || !arrivals)
         return;
-
-    const int row0 = (KSPLIT ? blockIdx.x : blockIdx.x * W) * kTileRows;
-    fused_reduction_tail(out, fused_out, M, NTOK, ldc, split_k, relu, row0, (KSPLIT ? 1 : W) * kTileRows,
-                         arrivals + blockIdx.x, reinterpret_cast<unsigned int*>(lds),
-                         W * kWave);
+    fused_reduction_tail(out, fused_out, M, NTOK, ldc, split_k, relu, blockIdx.x * kTileRows, kTileRows,
+                         arrivals + blockIdx.x, reinterpret_cast<unsigned int*>(lds), W * kWave);
 }
 
 // C[n][m] = fp16(sum over slabs of float(W[s][n][m])) (csrc/Reduction_Kernel.cuh:36-46), 8 elements
