@@ -496,6 +496,25 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
         for (int s = 0; s < 2; s++)
             b_off[c][s] = tok * 128 + (((s * 4 + q) ^ (tok & 7)) << 4);
     }
+    // ROWMAJ: the tile's 64 x N block sits in the wave's buffer as it sits in memory, row k at
+    // byte k * 2 N (with 64 tokens the four 32-byte column chunks of a row are permuted by
+    // (k >> 1) & 3, so that the four rows one transposing read touches fall into different
+    // banks).  ds_read_b64_tr_b16 hands lane i of a group of sixteen the i-th column of a 4 x 16
+    // block whose rows the sixteen lanes address four to a row: lane j points at row j / 4,
+    // columns 4 (j % 4) .. + 3.  Two such reads give a lane its eight consecutive k of one token.
+    auto rowmaj_byte = [](int k, int n) {
+        return NTOK == 64 ? k * 128 + ((((n >> 4) ^ (k >> 1)) & 3) << 5) + (n & 15) * 2 : (k * NTOK + n) * 2;
+    };
+    int tr_off[NB][2][2];
+    if (ROWMAJ) {
+#pragma unroll
+        for (int c = 0; c < NB; c++)
+#pragma unroll
+            for (int s = 0; s < 2; s++)
+#pragma unroll
+                for (int hh = 0; hh < 2; hh++)
+                    tr_off[c][s][hh] = rowmaj_byte(32 * s + 8 * q + 4 * hh + (l15 >> 2), (16 * c + 4 * (l15 & 3)) % NTOK);
+    }
     // BSW: load i of this wave's share of a tile covers tokens share0 + 8 i + (lane >> 3), lane & 7
     // being the 16-byte granule of the token's 128-byte line; lanes beyond the share (a share of
     // four tokens fills half a load) repeat a token and write nothing.
@@ -683,23 +702,32 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
             if (BLDS || ROWMAJ || BSW > 0) {
                 const uint8_t* bt = bslice + (BLDS ? (size_t)s.tile * (NTOK * 128) : BSW > 0 ? (s.tile & 1) * (NTOK * 128) : 0);
                 if (ROWMAJ) {
-                    // lane l of piece h holds tokens n0 .. n0+7 of row k, (k, n0) = divmod(512 h + 8 l, N);
-                    // element (k, n) goes to byte n*128 + (((k >> 3) ^ (n & 7)) << 4) + 2*(k & 7), n & 7 = j
+                    // lane l of piece h holds tokens n0 .. n0+7 of row k, (k, n0) = divmod(512 h + 8 l, N)
     #pragma unroll
                     for (int h = 0; h < BL; h++) {
                         const int e0 = h * 512 + lane * 8;
-                        const int k = e0 / NTOK, n0 = e0 % NTOK;
-                        const int base = n0 * 128 + (k & 7) * 2, g0 = (k >> 3) << 4;
-    #pragma unroll
-                        for (int j = 0; j < 8; j++)
-                            *reinterpret_cast<_Float16*>(bslice + ((g0 ^ (j << 4)) + base) + j * 128) = bfrag[slot][h][j];
+                        *reinterpret_cast<half8*>(bslice + rowmaj_byte(e0 / NTOK, e0 % NTOK)) = bfrag[slot][h];
                     }
+                    asm volatile("" ::: "memory");  // other lanes' reads below come after these writes
+                    typedef short short4v __attribute__((ext_vector_type(4)));
+                    typedef short short8v __attribute__((ext_vector_type(8)));
+                    typedef __attribute__((address_space(3))) short4v lds_short4v;
+    #pragma unroll
+                    for (int cb = 0; cb < NB; cb++)
+    #pragma unroll
+                        for (int k = 0; k < 2; k++) {
+                            const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v*)(bt + tr_off[cb][k][0]));
+                            const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v*)(bt + tr_off[cb][k][1]));
+                            const short8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                            bf[cb][k] = __builtin_bit_cast(half8, both);
+                        }
+                } else {
+    #pragma unroll
+                    for (int cb = 0; cb < NB; cb++)
+    #pragma unroll
+                        for (int k = 0; k < 2; k++)
+                            bf[cb][k] = *reinterpret_cast<const half8*>(bt + b_off[cb][k]);
                 }
-    #pragma unroll
-                for (int cb = 0; cb < NB; cb++)
-    #pragma unroll
-                    for (int k = 0; k < 2; k++)
-                        bf[cb][k] = *reinterpret_cast<const half8*>(bt + b_off[cb][k]);
             } else {
     #pragma unroll
                 for (int cb = 0; cb < NB; cb++)
