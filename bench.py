@@ -150,7 +150,10 @@ def events_ms(lib, sptr, call, n):
 
 
 SWEEP = [
-    # (label, workload, N, sparsity, row_skewed)
+    # (label, workload, N, sparsity, row_skewed); a label ending in _row_major goes through
+    # SpMM_SplitK_API_RowMajor (B[K][N], C[M][N]: this fork's own operand layout)
+    ("ffn1_n16_row_major", "opt30b_ffn1", 16, 0.8, False),
+    ("ffn1_n64_row_major", "opt30b_ffn1", 64, 0.8, False),
     ("ffn1_n8", "opt30b_ffn1", 8, 0.8, False),
     ("ffn1_n32", "opt30b_ffn1", 32, 0.8, False),
     ("ffn1_n64", "opt30b_ffn1", 64, 0.8, False),
@@ -195,16 +198,20 @@ def sweep(G, lib, torch, dev, sptr, with_stack):
         p_offs = [ctypes.c_void_p(t.data_ptr()) for t in d_offs]
         p_B, p_C, p_W = (ctypes.c_void_p(t.data_ptr()) for t in (d_B, d_C, d_W))
 
+        row_major = label.endswith("_row_major")  # the same buffers hold either layout's elements
+        entry = lib.SpMM_SplitK_API_RowMajor if row_major else lib.SpMM_SplitK_API
+
         def call(i):
-            rc = lib.SpMM_SplitK_API(sptr, None, p_items[i % copies], p_offs[i % copies], p_B, p_C, M, N, K, p_W, split_k)
+            rc = entry(sptr, None, p_items[i % copies], p_offs[i % copies], p_B, p_C, M, N, K, p_W, split_k)
             if rc:
-                raise RuntimeError(f"SpMM_SplitK_API -> {rc}")
+                raise RuntimeError(f"{'SpMM_SplitK_API_RowMajor' if row_major else 'SpMM_SplitK_API'} -> {rc}")
 
         prewarm(call, torch, 0.1)
         ms = float(np.median([events_ms(lib, sptr, call, 100) for _ in range(3)])) / 100
         torch.cuda.synchronize()
         plan = G.SpMM_PlanLaunch(M, N, K, split_k)
         out.append({"case": label, "M": M, "K": K, "N": N, "sparsity": sparsity, "row_skewed": skew, "split_k": split_k,
+                    "layout": "B[K][N], C[M][N]" if row_major else "B[N][K], C[N][M]",
                     "plan": f"mode {plan['mode']}, {plan['waves']} waves", "compressed_bytes": a_bytes,
                     "ms": ms, "frac": a_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                     "tflops": 2.0 * M * N * K / (ms * 1e-3) / 1e12})
