@@ -432,10 +432,12 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
         }
     };
 
-    // Pipeline, per unit u (records two units ahead, the tile one buffer ahead; queue oldest first):
-    //   in flight at the top        records(u), tile(u+1), records(u+1)
-    //   wait until only kLoadsA stay   -> records(u) and tile(u+1) have landed
-    //   tile(u+1) -> the other LDS buffer; issue tile(u+2), records(u+2); multiply unit u; barrier
+    // Pipeline, per unit u (records two units ahead, the tile one buffer ahead; queue oldest first;
+    // with the residual, "records" stands for records + words, and every unit's loads are led by
+    // the offsets of the unit after it):
+    //   in flight at the top        records(u), [offsets(u+2),] tile(u+1), records(u+1)
+    //   wait until only kLoadsA stay   -> records(u), offsets(u+2) and tile(u+1) have landed
+    //   tile(u+1) -> the other LDS buffer; issue [offsets(u+3),] tile(u+2), records(u+2); multiply unit u; barrier
     // Loads past the batch's end repeat its last unit, so every path issues the same loads and the
     // wait count is a constant.  A buffer is written only after the barrier that follows its last reader.
     UnitRegs x[3];
