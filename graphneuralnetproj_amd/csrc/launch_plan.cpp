@@ -193,7 +193,9 @@ LaunchPlan plan_launch(int M, int N, int K, int split_k, bool row_major, double*
 {
     // a measured optimum with this Split_K: of the weight's own density if the caller gave it, else of any
     if (const Tuned* t = find_tuned(M, N, K, split_k, tile_bytes > 0.0 ? density_table(tile_bytes) : -1)) {
-        LaunchPlan p{t->mode, t->waves, t->stage_b, 0};
+        // (row-major activations are not staged per batch: every wave keeps its own tile of them in
+        // LDS, and the row-sharing shapes measure as fast that way as the staged column-major ones)
+        LaunchPlan p{t->mode, t->waves, row_major ? 0 : t->stage_b, 0};
         if (complete_plan(N, K, split_k, row_major, p)) {
             if (cost_us)
                 *cost_us = plan_cost_us(M, N, K, split_k, p, tile_bytes);
@@ -215,7 +217,7 @@ LaunchPlan plan_launch(int M, int N, int K, int split_k, bool row_major, double*
                 // fragments from memory and 1, 2 or 4 waves above.
                 if (mode == 0 && (N <= 16 ? (!stage || w < 5) : (stage || (w != 1 && w != 2 && w != 4))))
                     continue;
-                LaunchPlan p{mode, w, stage, 0};
+                LaunchPlan p{mode, w, row_major ? 0 : stage, 0};
                 if (!complete_plan(N, K, split_k, row_major, p))
                     continue;
                 const double c = plan_cost_us(M, N, K, split_k, p, tile_bytes);
