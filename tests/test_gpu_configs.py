@@ -87,6 +87,38 @@ def test_feed_forward_sparsity_sweep(spmm, oracle, M, K, sparsity, skew):
                                     f"feed-forward {sparsity:.0%}{' skewed' if skew else ''}")
 
 
+@pytest.mark.parametrize("M,K,sparsity", [(28672, 7168, 0.8), (21504, 7168, 0.8), (7168, 28672, 0.9)])
+def test_row_major_entry_full_size(spmm, oracle, M, K, sparsity):
+    """The fork's own operand layout (B[K][N], C[M][N]) at real sizes, N in {8, 16, 32, 64}: the
+    K-splitting layout with one batch (FFN1), the row-sharing one (QKV) and split-K with the second
+    kernel (FFN2): sampled rows against the oracle and every element against the column-major entry."""
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    A = spmm.synth_weights(M, K, sparsity, False, seed=M // 64 + K + 3)
+    items, offsets = spmm.InitSparseMatrixA_API(A)
+    d_items = torch.from_numpy(items.view(np.int32)).to(dev)
+    d_offs = torch.from_numpy(offsets).to(dev)
+    rows = np.sort(np.random.default_rng(M + K).choice(M, size=96, replace=False))
+    for N in (8, 16, 32, 64):
+        split_k = spmm.SpMM_SuggestSplitK_Bytes(M, N, K, int(offsets[-1]))
+        B = spmm.synth_activations(N, K, seed=9 + N)
+        d_B = torch.from_numpy(B.view(np.int16).copy()).to(dev).view(torch.float16)
+        d_Bt = d_B.t().contiguous()
+        d_W = torch.full((max(split_k, 1), N, M), float("nan"), dtype=torch.float16, device=dev)
+        d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device=dev)
+        d_Ct = torch.full((M, N), float("nan"), dtype=torch.float16, device=dev)
+        print(f"[gpu case] row-major entry M={M} K={K} N={N} split_k={split_k} sparsity={sparsity}", flush=True)
+        spmm.SpMM_SplitK_API_RowMajor(torch.cuda.current_stream(), None, d_items, d_offs, d_Bt, d_Ct, M, N, K, d_W, split_k)
+        torch.cuda.synchronize()
+        spmm.SpMM_SplitK_API(torch.cuda.current_stream(), None, d_items, d_offs, d_B, d_C, M, N, K, d_W, split_k)
+        torch.cuda.synchronize()
+        Ct = d_Ct.cpu().numpy()
+        _close(Ct[rows].T, oracle.gemm_f32(np.ascontiguousarray(A[rows]), B))
+        C = d_C.cpu().numpy().astype(np.float32)
+        diff = np.abs(Ct.T.astype(np.float32) - C)   # same products, other summation order
+        assert (diff <= 2 * (ATOL + RTOL * np.abs(C))).all(), float(diff.max())
+
+
 def test_decoder_stack_64_layers_full_size(spmm, oracle):
     """64 OPT-66B-shaped blocks (h = 9216, 52 GB of Tiled-CSL resident), 16 tokens, one token step:
     finite output of sane magnitude, a captured HIP graph of the step replays the eager bits, and
