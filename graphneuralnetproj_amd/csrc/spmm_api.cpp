@@ -266,8 +266,7 @@ extern "C" int SpMM_SplitK_API_Planned(void* stream, const void* Compressed_A, c
 {
     tcsl::LaunchPlan p{Mode, Waves, StageB, 0};
     if (!tcsl::complete_plan(N, K > 0 ? K : 64, Split_K, RowMajor != 0, p) ||
-        (Flags & ~(SPMM_FLAG_RELU | SPMM_FLAG_SEPARATE_REDUCTION | SPMM_FLAG_ADAPTIVE_WAVES)) != 0 ||
-        (RowMajor && (Flags & SPMM_FLAG_RELU)))
+        (Flags & ~(SPMM_FLAG_RELU | SPMM_FLAG_SEPARATE_REDUCTION | SPMM_FLAG_ADAPTIVE_WAVES)) != 0)
         return tcsl_error_invalid_value();
     CallOptions o;
     o.relu = (Flags & SPMM_FLAG_RELU) != 0;
@@ -389,8 +388,8 @@ int spmm_splitk(void* stream, const void* Compressed_A, const int* TileOffsets, 
     } else {
         // Dense slabs of partial sums; stride and clamp are applied by the reduction, which the
         // main kernel does itself (its last workgroup per group of rows) unless the caller wants
-        // the main kernel timed alone, the operands are row-major, or no counters are free.
-        const bool want_fused = !o.row_major && !o.separate_reduction && !o.ev_begin && !o.ev_end;
+        // the main kernel timed alone or no counters are free.
+        const bool want_fused = !o.separate_reduction && !o.ev_begin && !o.ev_end;
         rc = launch_main(stream, Compressed_A, TileOffsets, B, Reduction_Workspace, M, N, K, Split_K, o, ldb, M, o.relu,
                          want_fused ? C : nullptr, ldc, &fused);
     }

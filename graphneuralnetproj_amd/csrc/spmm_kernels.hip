@@ -168,6 +168,11 @@ __device__ __forceinline__ void store_through(_Float16* p, half4 v)
     __hip_atomic_store(reinterpret_cast<uint64_t*>(p), __builtin_bit_cast(uint64_t, v), __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_SYSTEM);
 }
+__device__ __forceinline__ void store_through(_Float16* p, _Float16 v)
+{
+    __hip_atomic_store(reinterpret_cast<uint16_t*>(p), __builtin_bit_cast(uint16_t, v), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_SYSTEM);
+}
 __device__ __forceinline__ half8 load_through(const _Float16* p)
 {
     typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
@@ -237,9 +242,12 @@ __device__ __forceinline__ void clear_tile(uint8_t* tile, int lane)
 // number of threads of the workgroup that are still there (the first nthreads).
 // Bits 8 and up of `relu` count further slabs that an earlier launch on the same stream left right
 // behind this launch's own Split_K (the 2:4 part's partial sums); they are added after them.
+// row_major: slabs and C are [M][N] (the rows' block is one contiguous run of nrows * N values;
+// ldc is not used) instead of one M vector per token.
 __device__ __forceinline__ void fused_reduction_tail(const _Float16* __restrict__ slabs, _Float16* __restrict__ C, int M,
                                                      int N, int ldc, int split_k, int relu, int row0, int nrows,
-                                                     unsigned int* counter, unsigned int* flag, int nthreads)
+                                                     unsigned int* counter, unsigned int* flag, int nthreads,
+                                                     bool row_major)
 {
     // this workgroup's partial sums have reached memory before it is counted
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), on top of what the compiler tracks itself
@@ -256,7 +264,8 @@ __device__ __forceinline__ void fused_reduction_tail(const _Float16* __restrict_
     const size_t slab = (size_t)M * N;
     for (int c = threadIdx.x; c < per_tok * N; c += nthreads) {
         const int tok = c / per_tok, m8 = c - tok * per_tok;
-        const _Float16* w0 = slabs + (size_t)tok * M + row0 + m8 * 8;
+        const size_t at = row_major ? (size_t)row0 * N + (size_t)c * 8 : (size_t)tok * M + row0 + m8 * 8;
+        const _Float16* w0 = slabs + at;
         float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         int sidx = 0;
         for (; sidx + 4 <= split_k; sidx += 4) {
@@ -280,7 +289,7 @@ __device__ __forceinline__ void fused_reduction_tail(const _Float16* __restrict_
 #pragma unroll
         for (int j = 0; j < 8; j++)
             o[j] = static_cast<_Float16>(relu ? fmaxf(sum[j], 0.f) : sum[j]);
-        *reinterpret_cast<half8*>(C + (size_t)tok * ldc + row0 + m8 * 8) = o;
+        *reinterpret_cast<half8*>(C + (row_major ? at : (size_t)tok * ldc + row0 + m8 * 8)) = o;
     }
     if (threadIdx.x == 0)
         *counter = 0;  // ready for the next call
@@ -288,7 +297,7 @@ __device__ __forceinline__ void fused_reduction_tail(const _Float16* __restrict_
 
 // ldb = elements between two tokens' vectors in B, ldo = the same for the output (column-major
 // only; the slabs of partial sums use M); relu != 0 clamps the output at zero (final results only).
-// arrivals != nullptr (KSPLIT, Split_K > 1, column-major): `out` receives the slabs of partial sums
+// arrivals != nullptr (KSPLIT, Split_K > 1): `out` receives the slabs of partial sums
 // as usual, and the last workgroup to finish a tile row adds the slabs up into fused_out (token
 // stride ldc, clamped if relu) itself; arrivals are counted in arrivals[blockIdx.x] (device memory,
 // zero before the launch and after it).  The row-sharing layout always leaves the sum to the
@@ -868,8 +877,13 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
             if (!(HALF && l15 >= 8)) {
                 if (ROWMAJ) {
 #pragma unroll
-                    for (int i = 0; i < 4; i++)  // the 16 tokens of a row are adjacent
-                        oslab[(r * 16 + q * 4 + i) * NTOK + c * 16 + l15] = h[i];
+                    for (int i = 0; i < 4; i++) {  // the 16 tokens of a row are adjacent
+                        _Float16* dst = oslab + (r * 16 + q * 4 + i) * NTOK + c * 16 + l15;
+                        if (arrivals)
+                            store_through(dst, h[i]);
+                        else
+                            *dst = h[i];
+                    }
                 } else {  // the four q-lanes of a token cover 32 bytes
                     _Float16* dst = oslab + (size_t)(c * 16 + l15) * ldo + r * 16 + q * 4;
                     if (arrivals)
@@ -933,10 +947,10 @@ __global__ __launch_bounds__(MAXW* kWave) void tcsl_spmm_kernel(const int* __res
     };
     if (KSPLIT || active)
         write_out();
-    if (!KSPLIT || ROWMAJ || !arrivals)
+    if (!KSPLIT || !arrivals)
         return;
     fused_reduction_tail(out, fused_out, M, NTOK, ldc, split_k, relu, blockIdx.x * kTileRows, kTileRows,
-                         arrivals + blockIdx.x, reinterpret_cast<unsigned int*>(lds), W * kWave);
+                         arrivals + blockIdx.x, reinterpret_cast<unsigned int*>(lds), W * kWave, ROWMAJ);
 }
 
 // C[n][m] = fp16(sum over slabs of float(W[s][n][m])) (csrc/Reduction_Kernel.cuh:36-46), 8 elements
@@ -1096,7 +1110,7 @@ extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offs
     unsigned int* arrivals = nullptr;
     if (fuse_page >= 0) {
         const long groups = mode ? M / kTileRows : (M / kTileRows + waves - 1) / waves;
-        if ((fuse_page >= kCounterPages && fuse_page != kScratchPage) || groups > kCountersPerPage || row_major ||
+        if ((fuse_page >= kCounterPages && fuse_page != kScratchPage) || groups > kCountersPerPage || mode != 1 ||
             split_k + (relu >> 8) < 2 || !fused_out)
             return static_cast<int>(hipErrorInvalidValue);
         DeviceArrays a;

@@ -256,8 +256,8 @@ SPMM_EXPORT int SpMM_PlanLaunch(int M_Global, int N_Global, int K_Global, int Sp
  * hipErrorInvalidValue when the shape does not fit (Waves above 8, or 4 for N = 64;
  * StageB with Mode 1 or RowMajor, StageB = 1 with N > 16, StageB = 2 outside the shapes above;
  * more than 160 KiB of LDS).  RowMajor != 0 selects
- * the operand layout of SpMM_SplitK_API_RowMajor; Flags as for SpMM_SplitK_API_Strided (no
- * clamp with row-major operands).  No counterpart in the reference.
+ * the operand layout of SpMM_SplitK_API_RowMajor; Flags as for SpMM_SplitK_API_Strided.  No
+ * counterpart in the reference.
  */
 SPMM_EXPORT int SpMM_SplitK_API_Planned(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
                                         void* C, int M_Global, int N_Global, int K_Global, void* Reduction_Workspace,

@@ -491,6 +491,44 @@ def test_fused_reduction_matches_separate_kernel_bit_for_bit(spmm, oracle, M, K,
         assert_close(outs[2], np.maximum(ref, 0.0))
 
 
+@pytest.mark.parametrize("M,K,N,split_k,waves", [(1024, 1024, 16, 4, 4), (1024, 2048, 8, 3, 8), (1152, 1024, 32, 5, 5),
+                                                 (1024, 1024, 64, 2, 4), (7168, 7168, 16, 4, 5)])
+def test_row_major_fused_reduction_matches_separate_kernel_bit_for_bit(spmm, oracle, M, K, N, split_k, waves):
+    """The fork's layout (B[K][N], C[M][N]) in the K-splitting layout: the reduction inside the launch
+    and the second kernel give the same bits, with and without the clamp, on repeated calls."""
+    torch = _torch()
+    dev = torch.device("cuda:0")
+    A, B, items, offsets = make_case(spmm, M, K, N, 0.8, seed=M + 5 * K + N + split_k)
+    d_items = torch.from_numpy(items.view(np.int32).copy()).to(dev)
+    d_offs = torch.from_numpy(offsets.copy()).to(dev)
+    d_Bt = torch.from_numpy(np.ascontiguousarray(B.T).view(np.int16).copy()).to(dev)
+    outs = []
+    for flags in (0, spmm.SPMM_FLAG_SEPARATE_REDUCTION, spmm.SPMM_FLAG_RELU,
+                  spmm.SPMM_FLAG_RELU | spmm.SPMM_FLAG_SEPARATE_REDUCTION):
+        d_C = torch.full((M, N), float("nan"), dtype=torch.float16, device=dev)
+        d_W = torch.full((split_k, M, N), float("nan"), dtype=torch.float16, device=dev)
+        print(f"[gpu case] row-major fused-vs-separate M={M} N={N} K={K} split_k={split_k} waves={waves} flags={flags}", flush=True)
+        for _ in range(3):  # repeated calls: the arrival counters must come back to zero every time
+            spmm.SpMM_SplitK_API_Planned(torch.cuda.current_stream(), d_items, d_offs, d_Bt, d_C, M, N, K, d_W, split_k, 1, waves,
+                                         0, 1, flags)
+        torch.cuda.synchronize()
+        outs.append(d_C.cpu().numpy())
+    assert np.array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16))
+    assert np.array_equal(outs[2].view(np.uint16), outs[3].view(np.uint16))
+    if M * K <= 4 * 1024 * 1024:
+        ref = oracle.gemm_f32(A, B)
+        assert_close(outs[0].T, ref)
+        assert_close(outs[2].T, np.maximum(ref, 0.0))
+    # the library's own entry (its own launch shape) agrees too
+    d_C = torch.full((M, N), float("nan"), dtype=torch.float16, device=dev)
+    d_W = torch.full((split_k, M, N), float("nan"), dtype=torch.float16, device=dev)
+    spmm.SpMM_SplitK_API_RowMajor(torch.cuda.current_stream(), None, d_items, d_offs, d_Bt, d_C, M, N, K, d_W, split_k)
+    torch.cuda.synchronize()
+    got = d_C.cpu().numpy().astype(np.float32)
+    want = outs[0].astype(np.float32)
+    assert (np.abs(got - want) <= 2e-2 + 2e-2 * np.abs(want)).all()
+
+
 @pytest.mark.parametrize("mode,waves,stage_b", [(0, 7, 1), (0, 3, 0), (1, 8, 0), (1, 5, 0)])
 def test_fused_reduction_in_every_launch_shape(spmm, oracle, mode, waves, stage_b):
     torch = _torch()
