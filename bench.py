@@ -342,6 +342,23 @@ def stack_step(G, torch, dev, layers=64, h=9216, N=16, sparsity=0.8, split=False
         print(f"bench.py: graph capture of the stack failed: {e}", file=sys.stderr)
     weight_bytes = sum(L.bytes() for L in blocks)
     ms = min(eager_ms, graph_ms) if graph_ms else eager_ms
+    row_major_ms = None
+    if not split:  # the same weights with the activations in this fork's layout, [features][tokens]
+        del stack, g
+        stack = DS.Stack(G, torch, blocks, h, N, row_major=True)
+        stack.x[0].copy_(x0.t())
+        for _ in range(5):
+            stack.step(stream)
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            for _ in range(5):
+                stack.step(stream)
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) * 1e3 / 5)
+        row_major_ms = float(np.median(times))
+        g = None
     del stack, blocks, g
     torch.cuda.empty_cache()
     case = "decoder_stack" if sparsity == 0.8 and not split else f"decoder_stack_{int(sparsity * 100)}pct" + ("_split" if split else "")
@@ -349,6 +366,8 @@ def stack_step(G, torch, dev, layers=64, h=9216, N=16, sparsity=0.8, split=False
             "form": "2:4 records + residual lists, one launch per product" if split else "Tiled-CSL",
             "weights": "random-init per layer, drawn and encoded on the GPU", "resident_weight_bytes": weight_bytes,
             "ms": ms, "eager_ms": eager_ms, "graph_ms": graph_ms, "frac": weight_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "row_major_eager_ms": row_major_ms,
+            "row_major_frac": weight_bytes / (row_major_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS if row_major_ms else None,
             "hbm_floor_ms": weight_bytes / (HBM_PEAK_GBPS * 1e9) * 1e3, "build_s": build_s}
 
 

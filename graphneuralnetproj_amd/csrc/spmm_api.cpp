@@ -260,6 +260,18 @@ extern "C" int SpMM_SplitK_API_Strided(void* stream, const void* Compressed_A, c
     return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, o);
 }
 
+extern "C" int SpMM_SplitK_API_RowMajor_Flags(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
+                                              void* C, int M, int N, int K, void* Reduction_Workspace, int Split_K, int Flags)
+{
+    if ((Flags & ~(SPMM_FLAG_RELU | SPMM_FLAG_SEPARATE_REDUCTION)) != 0)
+        return tcsl_error_invalid_value();
+    CallOptions o;
+    o.row_major = true;
+    o.relu = (Flags & SPMM_FLAG_RELU) != 0;
+    o.separate_reduction = (Flags & SPMM_FLAG_SEPARATE_REDUCTION) != 0;
+    return spmm_splitk(stream, Compressed_A, TileOffsets, B, C, M, N, K, Reduction_Workspace, Split_K, o);
+}
+
 extern "C" int SpMM_SplitK_API_Planned(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
                                        void* C, int M, int N, int K, void* Reduction_Workspace, int Split_K, int Mode,
                                        int Waves, int StageB, int RowMajor, int Flags)

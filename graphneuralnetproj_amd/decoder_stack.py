@@ -125,22 +125,30 @@ def build_split_layer_on_device(G, torch, dev, h, N, sparsity, seed, weight_std=
 
 
 class Stack:
-    def __init__(self, G, torch, layers, h, N):
-        self.G, self.torch, self.layers, self.h, self.N = G, torch, layers, h, N
+    """row_major: every buffer holds [features][N] (this fork's operand layout) instead of one vector per
+    token; the output projection then reads the first h rows of the fused QKV result.  Tiled-CSL weights only."""
+
+    def __init__(self, G, torch, layers, h, N, row_major=False):
+        self.G, self.torch, self.layers, self.h, self.N, self.row_major = G, torch, layers, h, N, row_major
         first = layers[0].mats["qkv"]
         dev = (first[1][0] if Layer.is_split(first) else first[1]).device
         f16 = torch.float16
-        self.x = [torch.zeros((N, h), dtype=f16, device=dev) for _ in range(2)]  # ping-pong layer inputs
-        self.qkv = torch.zeros((N, 3 * h), dtype=f16, device=dev)
-        self.o = torch.zeros((N, h), dtype=f16, device=dev)
-        self.f = torch.zeros((N, 4 * h), dtype=f16, device=dev)
+        shape = (lambda rows: (rows, N)) if row_major else (lambda rows: (N, rows))
+        self.x = [torch.zeros(shape(h), dtype=f16, device=dev) for _ in range(2)]  # ping-pong layer inputs
+        self.qkv = torch.zeros(shape(3 * h), dtype=f16, device=dev)
+        self.o = torch.zeros(shape(h), dtype=f16, device=dev)
+        self.f = torch.zeros(shape(4 * h), dtype=f16, device=dev)
         max_split = max(1, max(s for L in layers for (_, _, _, _, s) in L.mats.values()))
         # one workspace for every product, as the reference's caller keeps (third_party/ft.patch:2762-2765)
         self.ws = torch.zeros((max_split, N, 4 * h), dtype=f16, device=dev)
 
     def _product(self, stream, mat, src, ldb, dst, ldc, flags=0):
         it, of, M, K, s = mat
-        if Layer.is_split(mat):
+        if self.row_major:
+            if Layer.is_split(mat) or it is None:
+                raise ValueError("the row-major chain takes Tiled-CSL weights only")
+            self.G.SpMM_SplitK_API_RowMajor_Flags(stream, it, of, src, dst, M, self.N, K, self.ws, s, flags)
+        elif Layer.is_split(mat):
             self.G.HeteroSparse_Fused_SpMM_API_Strided(stream, it[0], it[1], of[0], of[1], src, ldb, dst, ldc, M, self.N, K,
                                                        self.ws, s, flags)
         elif it is not None:
@@ -177,6 +185,8 @@ def main():
                     help="device: every layer's weights are drawn and encoded on the GPU (default); host: drawn and "
                          "encoded on the host by the library's generator and encoder; copied: one host-made layer, "
                          "copied in HBM for the others")
+    ap.add_argument("--row-major", action="store_true",
+                    help="keep the activations as [features][tokens] (this fork's layout) and use the row-major entry")
     ap.add_argument("--split", action="store_true",
                     help="split every weight into a 2:4 part and a residual and multiply both in one launch "
                          "(worth it up to about 70 %% sparsity); weights are made on the GPU")
@@ -213,8 +223,10 @@ def main():
                               else first.clone())
     torch.cuda.synchronize()
     prep_s = time.perf_counter() - t0
-    stack = Stack(G, torch, layers, h, N)
+    stack = Stack(G, torch, layers, h, N, row_major=args.row_major)
     x0 = torch.from_numpy(G.synth_activations(N, h, seed=99).view(np.int16)).to(dev).view(torch.float16)
+    if args.row_major:
+        x0 = x0.t().contiguous()
     stream = torch.cuda.current_stream()
 
     def run_eager():
@@ -266,6 +278,7 @@ def main():
         "config": {"workload": f"{args.layers} layers x (QKV, out-proj, FFN1+ReLU, FFN2), h={h}, N={N}, "
                                f"{args.sparsity * 100:.0f}% sparse",
                    "form": "2:4 records + residual lists, one launch per product" if args.split else "Tiled-CSL",
+                   "layout": "B[K][N], C[M][N]" if args.row_major else "B[N][K], C[N][M]",
                    "weights": "model directory" if args.model_dir else
                    {"device": "random-init per layer, drawn and encoded on the GPU",
                     "host": "random-init per layer, drawn and encoded on the host",

@@ -40,6 +40,7 @@ EXPORTED_SYMBOLS = (
     "SpMM_PlanLaunch",
     "SpMM_SplitK_API_Planned",
     "SpMM_SplitK_API_RowMajor",
+    "SpMM_SplitK_API_RowMajor_Flags",
     "SpMM_SplitK_API_Strided",
     "SpMM_DeviceEncodeOffsets",
     "SpMM_DeviceEncodeItems",
@@ -143,6 +144,9 @@ def load_library():
                                            ctypes.c_void_p]
     lib.SpMM_SplitK_API_RowMajor.restype = ctypes.c_int
     lib.SpMM_SplitK_API_RowMajor.argtypes = lib.SpMM_SplitK_API.argtypes
+    lib.SpMM_SplitK_API_RowMajor_Flags.restype = ctypes.c_int
+    lib.SpMM_SplitK_API_RowMajor_Flags.argtypes = [ctypes.c_void_p] * 5 + [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_int,
+                                                                                              ctypes.c_int]
     lib.SpMM_SynthWeights.restype = None
     lib.SpMM_SynthWeights.argtypes = [_u16p, ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_int,
                                       ctypes.c_uint64]
@@ -367,6 +371,20 @@ def SpMM_PlanLaunch(M_Global, N_Global, K_Global, Split_K):
         raise SpMMError("SpMM_PlanLaunch", rc)
     return {"mode": vals[0].value, "waves": vals[1].value, "stage_b": vals[2].value, "lds_bytes": vals[3].value,
             "estimated_us": est.value}
+
+
+def SpMM_SplitK_API_RowMajor_Flags(stream, Compressed_A, TileOffsets, B, C, M_Global, N_Global, K_Global, Reduction_Workspace,
+                                   Split_K, Flags=0):
+    """SpMM_SplitK_API_RowMajor (B[K][N], C[M][N]) with Flags (SPMM_FLAG_RELU, SPMM_FLAG_SEPARATE_REDUCTION)."""
+    lib = load_library()
+    if stream is not None and not isinstance(stream, int):
+        stream = stream.cuda_stream
+    rc = lib.SpMM_SplitK_API_RowMajor_Flags(ctypes.c_void_p(stream) if stream else None, _ptr(Compressed_A), _ptr(TileOffsets),
+                                            _ptr(B), _ptr(C), M_Global, N_Global, K_Global, _ptr(Reduction_Workspace), Split_K,
+                                            Flags)
+    if rc != 0:
+        raise SpMMError("SpMM_SplitK_API_RowMajor_Flags", rc, lib.SpMM_GetErrorString(rc).decode())
+    return rc
 
 
 def SpMM_SplitK_API_Planned(stream, Compressed_A, TileOffsets, B, C, M_Global, N_Global, K_Global,

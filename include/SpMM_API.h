@@ -151,6 +151,16 @@ SPMM_EXPORT int SpMM_SplitK_API_Strided(void* stream, const void* Compressed_A, 
                                         void* Reduction_Workspace, int Split_K, int Flags);
 
 /*
+ * SpMM_SplitK_API_RowMajor with the flags of SpMM_SplitK_API_Strided (the clamp, the reduction as a
+ * kernel of its own).  A chain of layers in this fork's layout needs no strides: a product's
+ * result C[M][N] is the next product's B[K][N] as it stands, and the output projection's input, the
+ * first third of the fused QKV result, is that result's first K rows.
+ */
+SPMM_EXPORT int SpMM_SplitK_API_RowMajor_Flags(void* stream, const void* Compressed_A, const int* TileOffsets, const void* B,
+                                               void* C, int M_Global, int N_Global, int K_Global, void* Reduction_Workspace,
+                                               int Split_K, int Flags);
+
+/*
  * SpMM_SplitK_API with two hipEvent_t recorded on `stream` immediately before and
  * after the main kernel (the split-K reduction, if any, follows KernelEnd), so a
  * benchmark can time that kernel alone inside its own loop.  Either event may be

@@ -459,6 +459,40 @@ def test_decoder_stack_matches_cpu_chain(spmm, oracle):
     assert (err <= 3 * (ATOL + RTOL * scale)).all(), err.max()
 
 
+def test_row_major_decoder_stack_matches_cpu_chain(spmm, oracle):
+    """The same three blocks with every buffer as [features][tokens] (the fork's layout): the output
+    projection reads the first h rows of the fused QKV result, the clamp rides on the row-major entry."""
+    torch = _torch()
+    from graphneuralnetproj_amd import decoder_stack as DS
+
+    dev = torch.device("cuda:0")
+    h, N, nlayers = 512, 16, 3
+    layers, dense = [], []
+    for i in range(nlayers):
+        L, d = DS.build_layer(spmm, torch, dev, h, N, 0.6, seed=40 + i, keep_dense=True, weight_scale=4.0)
+        layers.append(L)
+        dense.append(d)
+    stack = DS.Stack(spmm, torch, layers, h, N, row_major=True)
+    x0 = spmm.synth_activations(N, h, seed=99)
+    stack.x[0].copy_(torch.from_numpy(np.ascontiguousarray(x0.T).view(np.int16)).to(dev).view(torch.float16))
+    print(f"[gpu case] row-major decoder stack h={h} N={N} layers={nlayers}", flush=True)
+    out = stack.step(torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().T
+    x = x0
+    f16 = lambda a: a.astype(np.float16)
+    for d in dense:
+        qkv = f16(oracle.gemm_f32(d["qkv"], x))
+        o = f16(oracle.gemm_f32(d["out"], np.ascontiguousarray(qkv[:, :h])))
+        f = f16(np.maximum(oracle.gemm_f32(d["ffn1"], o), 0.0))
+        x = f16(oracle.gemm_f32(d["ffn2"], f))
+    xr = x.astype(np.float32)
+    assert np.abs(xr).max() > 1e-3
+    err = np.abs(got.astype(np.float32) - xr)
+    scale = np.maximum(np.abs(xr), np.sqrt(np.mean(xr * xr)))
+    assert (err <= 3 * (ATOL + RTOL * scale)).all(), err.max()  # as for the column-major chain
+
+
 @pytest.mark.parametrize("M,K,N,split_k", [
     (1024, 1024, 16, 4), (1024, 1024, 8, 2), (1024, 2048, 32, 8), (1024, 1024, 64, 3),
     (1152, 1024, 16, 5),      # nine tile rows: a partly filled workgroup in the row-sharing layout
