@@ -856,7 +856,7 @@ __global__ __launch_bounds__(64) void a24_residual_emit_kernel(const uint16_t* _
     const int begin = offsets[list];
     if (list == lists - 1)  // the padding behind the last list
         words[(size_t)offsets[lists] + L] = 0;
-    if (n == 0)
+    if (n == 0 || n > kMaxListWords)  // (more than a residual can hold: not this format's input; nothing is written)
         return;
     int at = incl - mine_n;
     const bool in_order = n <= 64;  // one round: the host leaves such a list as collected

@@ -579,6 +579,8 @@ def pack_residual_on_device(A2_d, stream=None):
     total, longest = (int(x) for x in offsets[lists:lists + 2].cpu())
     if total < 0:
         raise SpMMError("HeteroSparse_DevicePackA2_Offsets", -1, "more residual values than an int counts")
+    if longest > 1024:
+        raise SpMMError("HeteroSparse_DevicePackA2_Offsets", -1, "not a residual: a 16 x 128 block with more than 1024 kept values")
     words = torch.empty(total + 64, dtype=torch.int32, device=A2_d.device)
     rc = lib.HeteroSparse_DevicePackA2_Words(sp, _ptr(A2_d), M, K, _ptr(offsets), _ptr(words))
     if rc != 0:

@@ -402,8 +402,10 @@ SPMM_EXPORT int HeteroSparse_A1_Partials(void* stream, const void* Packed_A1, co
  *   HeteroSparse_DevicePackA2_Words    fills Words_d (T + 64 words, the last 64 zero) from A2_d and
  *                                      those offsets.
  * Both only enqueue kernels on `stream`; read T and the longest list back (after synchronising) to
- * size the second buffer, or allocate the worst case M*K/2 + 64 words up front.  Return a hipError_t
- * value; hipErrorInvalidValue for M % 128, K % 128 or null pointers.
+ * size the second buffer, or allocate the worst case M*K/2 + 64 words up front.  A2_d must be a
+ * residual: at most two kept values in every group of four, hence at most 1024 per 16 x 128 block
+ * (a block that holds more gets no words; *LongestList_d shows it).  Return a hipError_t value;
+ * hipErrorInvalidValue for M % 128, K % 128 or null pointers.
  */
 SPMM_EXPORT int HeteroSparse_DevicePackA2_Offsets(void* stream, const void* A2_d, int M_Global, int K_Global, int* Offsets_d,
                                                   int* LongestList_d);

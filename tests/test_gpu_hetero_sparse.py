@@ -620,3 +620,31 @@ def test_split_decoder_stack_matches_cpu_chain(spmm, oracle):
         torch.cuda.synchronize()
         assert torch.equal(out_g, got), f"replay {rep} differs from the eager result"
 
+
+def test_device_residual_lists_refuse_what_is_no_residual(spmm):
+    """A dense matrix has 2048 kept values per 16 x 128 block, twice what a residual can hold: the
+    offsets step reports it, the Python wrapper raises, and the words step writes nothing for such blocks."""
+    torch = _torch()
+    M, K = 128, 256
+    A = torch.ones((M, K), dtype=torch.float16, device="cuda:0")
+    with pytest.raises(spmm.SpMMError):
+        spmm.pack_residual_on_device(A)
+    lib = spmm.load_library()
+    import ctypes
+
+    lists = (M // 16) * (K // 128)
+    offsets = torch.zeros(lists + 2, dtype=torch.int32, device="cuda:0")
+    words = torch.full((lists * 2048 + 64,), 7, dtype=torch.int32, device="cuda:0")
+    print("[gpu case] device residual lists on a dense matrix", flush=True)
+    rc = lib.HeteroSparse_DevicePackA2_Offsets(None, ctypes.c_void_p(A.data_ptr()), M, K, ctypes.c_void_p(offsets.data_ptr()),
+                                               ctypes.c_void_p(offsets.data_ptr() + 4 * (lists + 1)))
+    assert rc == 0
+    rc = lib.HeteroSparse_DevicePackA2_Words(None, ctypes.c_void_p(A.data_ptr()), M, K, ctypes.c_void_p(offsets.data_ptr()),
+                                             ctypes.c_void_p(words.data_ptr()))
+    assert rc == 0
+    torch.cuda.synchronize()
+    o = offsets.cpu().numpy()
+    assert o[lists] == lists * 2048 and o[lists + 1] == 2048
+    w = words.cpu().numpy()
+    assert (w[:lists * 2048] == 7).all() and (w[lists * 2048:] == 0).all()  # only the padding was written
+
