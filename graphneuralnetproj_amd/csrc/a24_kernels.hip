@@ -17,6 +17,10 @@
 #include <mutex>
 #include <type_traits>
 
+#include "split_k_in_launch.h"
+
+extern "C" int tcsl_counter_page_address(int page, unsigned int** address);  // spmm_kernels.hip
+
 namespace {
 
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
@@ -251,7 +255,9 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
                                                                      _Float16* __restrict__ out, int units,
                                                                      int units_per_batch, long ldb, long ldo, long slab,
                                                                      int n_tokens, const unsigned* __restrict__ words,
-                                                                     const int* __restrict__ offsets, int relu)
+                                                                     const int* __restrict__ offsets, int relu, int M,
+                                                                     _Float16* __restrict__ fused_out,
+                                                                     unsigned int* __restrict__ arrivals, long ldc)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char tile[];  // [2][NT * 16][kRowBytes], then [W][kImageBytes]
     constexpr int kBuf = NT * 16 * kRowBytes;
@@ -531,19 +537,32 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
                 float4v s = acc[r][t];
                 if constexpr (RL > 0)
                     s += accd[r][t];
-                if (relu)
+                if (relu && !arrivals)  // partial sums are never clamped
                     s = float4v{fmaxf(s[0], 0.f), fmaxf(s[1], 0.f), fmaxf(s[2], 0.f), fmaxf(s[3], 0.f)};
                 half4 h = {static_cast<_Float16>(s[0]), static_cast<_Float16>(s[1]), static_cast<_Float16>(s[2]),
                            static_cast<_Float16>(s[3])};
-                *reinterpret_cast<half4*>(dstc + (size_t)n * ldo + (block0 + r) * 16 + (lane >> 4) * 4) = h;
+                _Float16* const to = dstc + (size_t)n * ldo + (block0 + r) * 16 + (lane >> 4) * 4;
+                if (arrivals)
+                    inlaunch::store_through(to, h);
+                else
+                    *reinterpret_cast<half4*>(to) = h;
             }
         }
     }
+    // arrivals != nullptr (more than one batch): `out` holds the batches' slabs ([N][M] each, M * N
+    // apart), and the last workgroup to finish this group of rows adds them up into fused_out (token
+    // stride ldc, clamped if relu), like the main kernel's K-splitting layout and with the same bits
+    // as the reduction kernel.
+    if (arrivals)
+        inlaunch::fused_reduction_tail(out, fused_out, M, n_tokens, static_cast<int>(ldc), gridDim.y, relu,
+                                       blockIdx.x * (16 * RB * W), 16 * RB * W, arrivals + blockIdx.x,
+                                       reinterpret_cast<unsigned int*>(tile), W * kWave, false);
 }
 
 template<int NT, int RB, int W, int RL>
 int launch_shared_b(hipStream_t stream, const void* packed, const void* B, void* out, int M, int N, int K, int split_k,
-                    long ldb, long ldo, long slab, const void* words, const void* offsets, int relu)
+                    long ldb, long ldo, long slab, const void* words, const void* offsets, int relu, void* fused_out,
+                    unsigned int* arrivals, long ldc)
 {
     const int units = K / 128;
     const int per_batch = (units + split_k - 1) / split_k;
@@ -558,7 +577,8 @@ int launch_shared_b(hipStream_t stream, const void* packed, const void* B, void*
     }
     hipLaunchKernelGGL(kern, dim3(M / (16 * RB * W), split_k), dim3(W * kWave), lds, stream,
                        static_cast<const uint8_t*>(packed), static_cast<const _Float16*>(B), static_cast<_Float16*>(out), units,
-                       per_batch, ldb, ldo, slab, N, static_cast<const unsigned*>(words), static_cast<const int*>(offsets), relu);
+                       per_batch, ldb, ldo, slab, N, static_cast<const unsigned*>(words), static_cast<const int*>(offsets), relu, M,
+                       static_cast<_Float16*>(fused_out), arrivals, ldc);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -566,11 +586,13 @@ int launch_shared_b(hipStream_t stream, const void* packed, const void* B, void*
 // shapes only: two row blocks per wave, four or eight waves.
 template<int NT>
 int launch_shared_b_nt(hipStream_t s, const void* packed, const void* B, void* out, int M, int N, int K, int split_k, int rb,
-                       int waves, long ldb, long ldo, long slab, int rl, const void* words, const void* offsets, int relu)
+                       int waves, long ldb, long ldo, long slab, int rl, const void* words, const void* offsets, int relu,
+                       void* fused_out, unsigned int* arrivals, long ldc)
 {
 #define A24_CASE(RB_, W_, RL_)                   \
     if (rb == RB_ && waves == W_ && rl == RL_) \
-        return launch_shared_b<NT, RB_, W_, RL_>(s, packed, B, out, M, N, K, split_k, ldb, ldo, slab, words, offsets, relu);
+        return launch_shared_b<NT, RB_, W_, RL_>(s, packed, B, out, M, N, K, split_k, ldb, ldo, slab, words, offsets, relu, \
+                                                 fused_out, arrivals, ldc);
     A24_CASE(2, 4, 0) A24_CASE(2, 8, 0)
     A24_CASE(2, 4, 1) A24_CASE(2, 8, 1) A24_CASE(2, 4, 2) A24_CASE(2, 8, 2) A24_CASE(2, 4, 3) A24_CASE(2, 8, 3)
     A24_CASE(2, 4, 4) A24_CASE(2, 4, 5) A24_CASE(2, 8, 4)
@@ -623,17 +645,31 @@ int launch_nt(hipStream_t s, const void* packed, const void* B, void* out, int M
 // residual_loads > 0 (share_b with rb == 2 only): the launch also multiplies the residual lists
 // words / offsets, none longer than 64 * residual_loads words.  relu (share_b only): negative
 // results are written as zero (for a launch that writes the finished result).
+// fuse_page >= 0 (share_b, split_k > 1, ldo == M, slab == M * N): the launch adds its slabs up into
+// fused_out (token stride ldc) itself, counting arrivals on that page of the library's counters.
 extern "C" int a24_launch_spmm(void* stream, const void* packed, const void* B, void* out, int M, int N, int K,
                                int split_k, int rb, int waves, int share_b, long ldb, long ldo, long slab,
-                               int residual_loads, const void* words, const void* offsets, int relu)
+                               int residual_loads, const void* words, const void* offsets, int relu, int fuse_page,
+                               void* fused_out, long ldc)
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
+    unsigned int* arrivals = nullptr;
+    if (fuse_page >= 0) {
+        if (!share_b || split_k < 2 || !fused_out || ldo != M || slab != static_cast<long>(M) * N || rb < 1 || waves < 1
+            || M / (16 * rb * waves) > 4096)
+            return static_cast<int>(hipErrorInvalidValue);
+        if (const int rc = tcsl_counter_page_address(fuse_page, &arrivals))
+            return rc;
+    }
     if (share_b) {  // waves own rows and share the activation tile through LDS
         switch (N) {
             case 8:
-            case 16: return launch_shared_b_nt<1>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets, relu);
-            case 32: return launch_shared_b_nt<2>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets, relu);
-            case 64: return launch_shared_b_nt<4>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets, relu);
+            case 16: return launch_shared_b_nt<1>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets, relu,
+                                                     fused_out, arrivals, ldc);
+            case 32: return launch_shared_b_nt<2>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets, relu,
+                                                     fused_out, arrivals, ldc);
+            case 64: return launch_shared_b_nt<4>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets, relu,
+                                                     fused_out, arrivals, ldc);
             default: return static_cast<int>(hipErrorInvalidValue);
         }
     }

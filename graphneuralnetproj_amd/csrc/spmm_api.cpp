@@ -23,7 +23,8 @@ int tcsl_launch_encode_offsets(void* stream, const void* A, int M, int K, int* o
 int tcsl_launch_encode_items(void* stream, const void* A, int M, int K, const int* offsets, void* items);
 int a24_launch_spmm(void* stream, const void* packed, const void* B, void* out, int M, int N, int K, int split_k, int rb,
                     int waves, int share_b, long ldb, long ldo, long slab, int residual_loads = 0,
-                    const void* words = nullptr, const void* offsets = nullptr, int relu = 0);
+                    const void* words = nullptr, const void* offsets = nullptr, int relu = 0, int fuse_page = -1,
+                    void* fused_out = nullptr, long ldc = 0);
 int a24_launch_split_pack(void* stream, const void* A, void* packed, void* residual, int M, int K);
 int a24_launch_residual_offsets(void* stream, const void* A2, int M, int K, int* offsets, int* longest);
 int a24_launch_residual_words(void* stream, const void* A2, int M, int K, const int* offsets, void* words);
@@ -563,6 +564,12 @@ bool a24_shape_ok(int M, int N, int K, int split_k, int row_blocks, int waves, i
 
 }  // namespace
 
+namespace {
+int a24_split_call(void* stream, const void* Packed_A1, const void* B, long ldb, void* C, long ldc, int M, int N, int K,
+                   void* Reduction_Workspace, int Split_K, int row_blocks, int waves, int loads, const void* words,
+                   const void* offsets, int relu, bool separate_reduction);
+}
+
 extern "C" int HeteroSparse_A1_Partials(void* stream, const void* Packed_A1, const void* B, void* Partials, int M, int N,
                                         int K, int Split_K, int RowBlocks, int Waves, int ShareB)
 {
@@ -614,6 +621,9 @@ extern "C" int HeteroSparse_SpMM_API(void* stream, const void* Packed_A1, const 
     int rc = 0;
     uint16_t* ws = static_cast<uint16_t*>(Reduction_Workspace);
     if (!residual) {
+        if (d.share_b)
+            return a24_split_call(stream, Packed_A1, B, K, C, M, M, N, K, ws, Split_K_A1, d.row_blocks, d.waves, 0, nullptr, nullptr,
+                                  0, false);
         rc = a24_launch_spmm(stream, Packed_A1, B, ws, M, N, K, Split_K_A1, d.row_blocks, d.waves, d.share_b, K, M, mn);
         return rc != 0 ? rc : tcsl_launch_reduce(stream, C, ws, mn, 1, mn, Split_K_A1, 0);
     }
@@ -684,6 +694,33 @@ extern "C" int HeteroSparse_DevicePackA2_Words(void* stream, const void* A2_d, i
 
 namespace {
 
+// The 2:4 kernel in its shared-tile layout with more than one batch, through to the finished C:
+// the launch sums its own slabs where a page of arrival counters can be had (and the caller does
+// not ask for the second kernel), else the reduction kernel follows.
+int a24_split_call(void* stream, const void* Packed_A1, const void* B, long ldb, void* C, long ldc, int M, int N, int K,
+                   void* Reduction_Workspace, int Split_K, int row_blocks, int waves, int loads, const void* words,
+                   const void* offsets, int relu, bool separate_reduction)
+{
+    const long mn = static_cast<long>(M) * N;
+    int page = -1;
+    std::unique_lock<std::mutex> page_lock;
+    // (up to 16 tokens: with more, the slabs' trip through memory inside the launch costs more than
+    // the second kernel: 9216 x 9216 at 60 % sparsity and N = 64 39.8 us against 35.2)
+    if (!separate_reduction && N <= 16 && M / (16 * row_blocks * waves) <= 4096) {
+        page_lock = std::unique_lock<std::mutex>(counter_pages().mutex());
+        page = counter_page(stream);
+    }
+    int rc = a24_launch_spmm(stream, Packed_A1, B, Reduction_Workspace, M, N, K, Split_K, row_blocks, waves, 1, ldb, M, mn, loads,
+                             words, offsets, page >= 0 ? relu : 0, page, page >= 0 ? C : nullptr, ldc);
+    if (rc == 0 && tcsl::CounterPages::recycled(page))
+        rc = tcsl_page_mark(page, stream);
+    if (page_lock.owns_lock())
+        page_lock.unlock();
+    if (rc != 0 || page >= 0)
+        return rc;
+    return tcsl_launch_reduce(stream, C, static_cast<uint16_t*>(Reduction_Workspace), M, N, ldc, Split_K, relu);
+}
+
 int fused_call(const char* who, void* stream, const void* Packed_A1, const void* A2_Words, const int* A2_Offsets, int LongestList,
                const void* B, long ldb, void* C, long ldc, int M, int N, int K, void* Reduction_Workspace, int Split_K, int Flags)
 {
@@ -696,7 +733,7 @@ int fused_call(const char* who, void* stream, const void* Packed_A1, const void*
     const int waves = (N == 64 && loads >= 5) ? 4 : a24_waves_for(M > 0 ? M : 128, Split_K);  // the former: what fits the registers
     if (!Packed_A1 || !A2_Words || !A2_Offsets || !B || !C || LongestList < 0 || LongestList > HETERO_FUSED_MAX_LIST
         || !a24_shape_ok(M, N, K, Split_K, 2, waves, 1) || (Split_K > 1 && !Reduction_Workspace) || ldb < K || ldc < M
-        || ldb % 8 != 0 || ldc % 8 != 0 || (Flags & ~SPMM_FLAG_RELU)) {
+        || ldb % 8 != 0 || ldc % 8 != 0 || (Flags & ~(SPMM_FLAG_RELU | SPMM_FLAG_SEPARATE_REDUCTION))) {
         std::fprintf(stderr, "%s: unsupported call M=%d N=%d K=%d Split_K=%d LongestList=%d ldb=%ld ldc=%ld (need M %% 128 == 0, K %% 128 == 0, no empty batch, lists of at most %d words, strides that are multiples of 8 and hold a vector, non-null pointers)\n",
                      who, M, N, K, Split_K, LongestList, ldb, ldc, HETERO_FUSED_MAX_LIST);
         return tcsl_error_invalid_value();
@@ -705,11 +742,8 @@ int fused_call(const char* who, void* stream, const void* Packed_A1, const void*
     const long mn = static_cast<long>(M) * N;
     if (Split_K == 1)
         return a24_launch_spmm(stream, Packed_A1, B, C, M, N, K, 1, 2, waves, 1, ldb, ldc, mn, loads, A2_Words, A2_Offsets, relu);
-    const int rc = a24_launch_spmm(stream, Packed_A1, B, Reduction_Workspace, M, N, K, Split_K, 2, waves, 1, ldb, M, mn, loads,
-                                   A2_Words, A2_Offsets, 0);
-    if (rc != 0)
-        return rc;
-    return tcsl_launch_reduce(stream, C, static_cast<uint16_t*>(Reduction_Workspace), M, N, ldc, Split_K, relu);
+    return a24_split_call(stream, Packed_A1, B, ldb, C, ldc, M, N, K, Reduction_Workspace, Split_K, 2, waves, loads, A2_Words,
+                          A2_Offsets, relu, (Flags & SPMM_FLAG_SEPARATE_REDUCTION) != 0);
 }
 
 }  // namespace

@@ -648,3 +648,36 @@ def test_device_residual_lists_refuse_what_is_no_residual(spmm):
     w = words.cpu().numpy()
     assert (w[:lists * 2048] == 7).all() and (w[lists * 2048:] == 0).all()  # only the padding was written
 
+
+@pytest.mark.parametrize("M,K,N,split_k", [(512, 1152, 16, 3), (384, 1152, 8, 2), (1024, 2048, 32, 4), (512, 1024, 64, 2),
+                                           (7168, 7168, 16, 4)])
+def test_fused_call_sums_its_slabs_in_the_launch_bit_for_bit(spmm, oracle, M, K, N, split_k):
+    """More than one batch: the 2:4 kernel's own sum of its slabs (the last workgroup of a group of rows)
+    and the reduction kernel give the same bits, with and without the clamp, on repeated calls; and
+    the call without a residual (HeteroSparse_SpMM_API on a 2:4 weight) goes the same way."""
+    torch = _torch()
+    A = spmm.synth_weights(M, K, 0.6, False, seed=M + K + N)
+    A1, A2 = spmm.HeteroSparse_Decompose(A)
+    words, offs, longest = spmm.HeteroSparse_PackA2(A2)
+    d_p, d_w, d_o = _dev(spmm.HeteroSparse_PackA1(A1)), _dev(words), _dev(offs)
+    Bh = spmm.synth_activations(N, K, seed=63)
+    d_B = _dev(Bh)
+    outs = []
+    for flags in (0, spmm.SPMM_FLAG_SEPARATE_REDUCTION, spmm.SPMM_FLAG_RELU, spmm.SPMM_FLAG_RELU | spmm.SPMM_FLAG_SEPARATE_REDUCTION):
+        d_C = torch.full((N, M), float("nan"), dtype=torch.float16, device="cuda:0")
+        d_W = torch.full((split_k, N, M), float("nan"), dtype=torch.float16, device="cuda:0")
+        print(f"[gpu case] one launch, slabs summed in the launch or not: M={M} N={N} K={K} split_k={split_k} flags={flags}", flush=True)
+        for _ in range(3):  # the arrival counters must come back to zero every time
+            spmm.HeteroSparse_Fused_SpMM_API_Strided(torch.cuda.current_stream(), d_p, d_w, d_o, longest, d_B, K, d_C, M, M, N, K,
+                                                     d_W, split_k, flags)
+        torch.cuda.synchronize()
+        outs.append(d_C.cpu().numpy())
+    assert np.array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16))
+    assert np.array_equal(outs[2].view(np.uint16), outs[3].view(np.uint16))
+    if M * K <= 4 * 1024 * 1024:
+        ref = oracle.gemm_f32(A, Bh)
+        assert_close(outs[0], ref)
+        assert_close(outs[2], np.maximum(ref, 0.0))
+        C1 = run_hybrid(spmm, spmm.HeteroSparse_PackA1(A1), None, None, Bh, M, N, K, split_k, 0)
+        assert_close(C1, oracle.gemm_f32(A1, Bh))
+
