@@ -422,7 +422,9 @@ SPMM_EXPORT int HeteroSparse_Fused_SpMM_API(void* stream, const void* Packed_A1,
 /*
  * HeteroSparse_Fused_SpMM_API for activations and results inside wider per-token buffers
  * (B[n*ldb + k], C[n*ldc + m], ldb >= K, ldc >= M, multiples of 8 elements) with an optional clamp
- * (Flags = 0 or SPMM_FLAG_RELU), like SpMM_SplitK_API_Strided: what a chain of decoder layers needs.
+ * (Flags = 0 or a sum of SPMM_FLAG_RELU and SPMM_FLAG_SEPARATE_REDUCTION), like SpMM_SplitK_API_Strided:
+ * what a chain of decoder layers needs.  With Split_K > 1 and up to 16 tokens the launch adds its
+ * slabs up itself (same bits as the reduction kernel, which SPMM_FLAG_SEPARATE_REDUCTION asks for).
  */
 SPMM_EXPORT int HeteroSparse_Fused_SpMM_API_Strided(void* stream, const void* Packed_A1, const void* A2_Words,
                                                     const int* A2_Offsets, int LongestList, const void* B, long ldb, void* C,
