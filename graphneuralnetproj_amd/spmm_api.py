@@ -84,7 +84,7 @@ def build_library():
     """Compile the library in-tree with hipcc (always recompiles)."""
     csrc = os.path.join(_PKG, "csrc")
     subprocess.run(["make", "-s", "-C", csrc, "clean"], check=True)
-    subprocess.run(["make", "-s", "-C", csrc, "-j4"], check=True)
+    subprocess.run(["make", "-s", "-C", csrc, "-j8"], check=True)
     return _LIB_PATH
 
 
