@@ -656,7 +656,7 @@ extern "C" int a24_launch_spmm(void* stream, const void* packed, const void* B, 
     unsigned int* arrivals = nullptr;
     if (fuse_page >= 0) {
         if (!share_b || split_k < 2 || !fused_out || ldo != M || slab != static_cast<long>(M) * N || rb < 1 || waves < 1
-            || M / (16 * rb * waves) > 4096)
+            || M / (16 * rb * waves) > 4096 || M % 8 != 0)
             return static_cast<int>(hipErrorInvalidValue);
         if (const int rc = tcsl_counter_page_address(fuse_page, &arrivals))
             return rc;
@@ -890,8 +890,11 @@ __global__ __launch_bounds__(64) void a24_residual_emit_kernel(const uint16_t* _
     }
     const int n = __shfl(incl, 63);
     const int begin = offsets[list];
+    const int total = offsets[lists];
+    if (total < 0)  // the word count did not fit an int: no offset of this table means anything, nothing is written
+        return;
     if (list == lists - 1)  // the padding behind the last list
-        words[(size_t)offsets[lists] + L] = 0;
+        words[(size_t)total + L] = 0;
     if (n == 0 || n > kMaxListWords)  // (more than a residual can hold: not this format's input; nothing is written)
         return;
     int at = incl - mine_n;
@@ -1033,6 +1036,13 @@ extern "C" int a24_side_begin(void* stream, void** side)
                 || hipEventCreateWithFlags(&n.fork, hipEventDisableTiming) != hipSuccess
                 || hipEventCreateWithFlags(&n.join, hipEventDisableTiming) != hipSuccess) {
                 (void)hipGetLastError();
+                // whatever was made before the failure goes back: the next call tries afresh
+                if (n.join)
+                    (void)hipEventDestroy(n.join);
+                if (n.fork)
+                    (void)hipEventDestroy(n.fork);
+                if (n.side)
+                    (void)hipStreamDestroy(n.side);
             } else {
                 side_table[side_used] = n;
                 e = &side_table[side_used++];

@@ -2,6 +2,15 @@
 
 namespace tcsl {
 
+void* CounterPages::stream_key(void* stream)
+{
+    if (reinterpret_cast<uintptr_t>(stream) != kPerThreadHandle)
+        return stream;
+    // thread-local storage is no address a stream handle (a heap object of the runtime) can have
+    thread_local char token;
+    return &token;
+}
+
 int CounterPages::acquire(void* stream, bool capturing, unsigned long long capture_id, IdleFn idle)
 {
     if (capturing) {

@@ -14,6 +14,12 @@
 // that the caller records behind every launch on such a page; a stream handle is never handed
 // back to the runtime by this class or on its behalf (the stream may long have been destroyed).
 // When nothing can be had the caller runs the reduction as a kernel of its own.
+//
+// The per-thread default stream is one handle value for every host thread but a different stream
+// in each: a call on it is keyed by (handle, calling thread), see stream_key().
+// What the scheme cannot see: a stream destroyed while its last launch is still running, and
+// another stream then created at the same handle address (a permanent page has no event to ask).
+// Callers that destroy streams with work in flight must synchronise them first.
 #pragma once
 
 #include <cstdint>
@@ -38,6 +44,13 @@ public:
     // from before this call until its launch has been enqueued and, if recycled(page), the
     // page's event recorded behind it, so that a page cannot change hands in between.
     int acquire(void* stream, bool capturing, unsigned long long capture_id, IdleFn idle);
+
+    // What names the stream of a call for acquire(): the handle itself, except for the per-thread
+    // default stream (handle value kPerThreadHandle in every host thread, a different stream in
+    // each), for which it is an address private to the calling thread.  Two host threads that
+    // launch on "the" per-thread stream at the same time therefore count on different pages.
+    static constexpr uintptr_t kPerThreadHandle = 2;  // hipStreamPerThread
+    static void* stream_key(void* stream);
 
     // Pages whose every launch must be followed by the event that `idle` looks at.
     static constexpr bool recycled(int page) { return page >= kPermanentPages && page < kEagerPages; }

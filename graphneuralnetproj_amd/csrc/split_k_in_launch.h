@@ -47,17 +47,25 @@ __device__ __forceinline__ half8 load_through(const _Float16* p)
 // behind this launch's own Split_K (the 2:4 part's partial sums); they are added after them.
 // row_major: slabs and C are [M][N] (the rows' block is one contiguous run of nrows * N values;
 // ldc is not used) instead of one M vector per token.
+// The sum moves eight rows at a time: nrows, M and row0 must be multiples of 8 (the launchers check M).
 __device__ __forceinline__ void fused_reduction_tail(const _Float16* __restrict__ slabs, _Float16* __restrict__ C, int M,
                                                      int N, int ldc, int split_k, int relu, int row0, int nrows,
                                                      unsigned int* counter, unsigned int* flag, int nthreads,
                                                      bool row_major)
 {
-    // this workgroup's partial sums have reached memory before it is counted
+    // This workgroup's partial sums have reached memory before it is counted.  The hardware side
+    // of that is the wait (the write-through stores are acknowledged at the coherence point); the
+    // two workgroup-scope fences say the same to the compiler, which may then move neither the
+    // slab stores below the counting nor the slab loads above it.  At workgroup scope a fence is
+    // waits only: no cache is written back or invalidated (a wider fence would flush the L2 that
+    // the weight stream lives in).
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), on top of what the compiler tracks itself
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
     if (threadIdx.x == 0)
         *flag = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     if (*flag != static_cast<unsigned int>(split_k - 1))
         return;
     split_k += relu >> 8;

@@ -128,7 +128,7 @@ int counter_page(void* stream)
     const int capturing = tcsl_stream_capture(stream, &capture_id);
     if (capturing < 0)
         return -1;
-    const int page = counter_pages().acquire(stream, capturing == 1, capture_id, [](int p) { return tcsl_page_idle(p) == 1; });
+    const int page = counter_pages().acquire(tcsl::CounterPages::stream_key(stream), capturing == 1, capture_id, [](int p) { return tcsl_page_idle(p) == 1; });
     // a page that changes hands is guarded by an event behind each of its launches; without one, no page
     if (page >= 0 && tcsl::CounterPages::recycled(page) && tcsl_page_prepare(page) != 0)
         return -1;

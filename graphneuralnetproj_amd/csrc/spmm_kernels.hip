@@ -1030,7 +1030,7 @@ extern "C" int tcsl_launch_spmm(void* stream, const void* items, const int* offs
     unsigned int* arrivals = nullptr;
     if (fuse_page >= 0) {
         const long groups = mode ? M / kTileRows : (M / kTileRows + waves - 1) / waves;
-        if ((fuse_page >= kCounterPages && fuse_page != kScratchPage) || groups > kCountersPerPage || mode != 1 ||
+        if ((fuse_page >= kCounterPages && fuse_page != kScratchPage) || groups > kCountersPerPage || mode != 1 || M % 8 != 0 ||
             split_k + (relu >> 8) < 2 || !fused_out)
             return static_cast<int>(hipErrorInvalidValue);
         DeviceArrays a;
@@ -1183,11 +1183,19 @@ extern "C" int tcsl_page_idle(int page)
         return 0;
     if (!page_guards[page].event)
         return 1;
+    // Asking an event is a call that the runtime forbids while any thread records a graph in the
+    // global capture mode (it would invalidate that capture), unless the asking thread's own mode
+    // is the relaxed one: switch to it for the one call.
+    hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+    if (hipThreadExchangeStreamCaptureMode(&mode) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;  // cannot ask safely: the page counts as busy
+    }
     const hipError_t e = hipEventQuery(page_guards[page].event);
-    if (e == hipSuccess)
-        return 1;
-    (void)hipGetLastError();
-    return 0;
+    if (e != hipSuccess)
+        (void)hipGetLastError();
+    (void)hipThreadExchangeStreamCaptureMode(&mode);  // back to what it was
+    return e == hipSuccess ? 1 : 0;
 }
 
 // Timing events for benchmarks (the host logic never includes HIP headers).

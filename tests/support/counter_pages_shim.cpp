@@ -26,7 +26,9 @@ int cp_acquire(void* p, unsigned long stream, int capturing, unsigned long long 
 {
     tcsl::CounterPages* pages = static_cast<tcsl::CounterPages*>(p);
     std::lock_guard<std::mutex> lock(pages->mutex());
-    const int page = pages->acquire(reinterpret_cast<void*>(stream), capturing != 0, capture_id, idle);
+    // the key the library derives from the handle (the per-thread default stream: one per calling thread)
+    void* key = tcsl::CounterPages::stream_key(reinterpret_cast<void*>(stream));
+    const int page = pages->acquire(key, capturing != 0, capture_id, idle);
     if (page >= 0)
         last_user[page] = reinterpret_cast<void*>(stream);
     return page;
@@ -37,5 +39,6 @@ int cp_eager_pages() { return tcsl::CounterPages::kEagerPages; }
 int cp_permanent_pages() { return tcsl::CounterPages::kPermanentPages; }
 int cp_recycled(int page) { return tcsl::CounterPages::recycled(page) ? 1 : 0; }
 int cp_capture_pages() { return tcsl::CounterPages::kCapturePages; }
+unsigned long cp_per_thread_handle() { return tcsl::CounterPages::kPerThreadHandle; }
 int cp_eviction_tries() { return tcsl::CounterPages::kEvictionTries; }
 }

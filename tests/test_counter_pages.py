@@ -130,3 +130,36 @@ def test_captures_have_their_own_pages_for_good(cp, pages):
     assert cp.cp_capture_in_use(pages) == C
     assert cp.cp_acquire(pages, s, 1, 5000) == -1
     assert cp.cp_acquire(pages, s, 1, 12) == b
+
+
+def test_per_thread_default_stream_is_one_stream_per_host_thread(cp, pages):
+    """hipStreamPerThread is a single handle value that names a different stream in every host
+    thread: launches from two threads may overlap, so they must not count on one page, while an
+    ordinary handle is the same stream whoever launches on it."""
+    import threading
+
+    cp.cp_per_thread_handle.restype = ctypes.c_ulong
+    h = cp.cp_per_thread_handle()
+    got = {}
+    gate = threading.Barrier(3)  # all three threads alive at once: their thread-local storage is distinct
+
+    def worker(name):
+        first = cp.cp_acquire(pages, h, 0, 0)
+        gate.wait()
+        got[name] = (first, cp.cp_acquire(pages, h, 0, 0), cp.cp_acquire(pages, stream(5), 0, 0),
+                     cp.cp_acquire(pages, h, 1, 77))
+        gate.wait()
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(3)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    firsts = [got[i][0] for i in range(3)]
+    assert len(set(firsts)) == 3 and min(firsts) >= 0          # one page per calling thread
+    assert all(got[i][1] == got[i][0] for i in range(3))       # and the thread keeps it
+    assert len({got[i][2] for i in range(3)}) == 1             # an ordinary handle: one stream, one page
+    captures = [got[i][3] for i in range(3)]                   # captures on it are per thread as well
+    assert len(set(captures)) == 3 and min(captures) >= cp.cp_eager_pages()
+    # the main thread's per-thread stream is yet another one
+    assert cp.cp_acquire(pages, h, 0, 0) not in firsts
