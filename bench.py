@@ -22,9 +22,18 @@ Prints ONE JSON line:
   cpu_baseline    the CPU path timed on this host: reference encoder (oracle/_ref,
                   single thread) + fp32-accumulate dense GEMM (oracle, single thread)
   sweep           the benchmark's other configurations, each timed for a fraction of a
-                  second after the headline (events around whole calls): ms per call and
-                  the fraction of 8 TB/s on that weight's compressed bytes; last, the
-                  64-layer decoder stack's time per token step
+                  second after the headline: ms per whole call (events around 100 calls) and
+                  the fraction of 8 TB/s on that weight's compressed bytes; kernel_ms, the main
+                  kernel alone writing C or its slabs of partial sums (events around 100
+                  launches of SpMM_SplitK_Partials); traffic where a counter profile of the
+                  case is kept under profiles/.  Covers N, sparsity and skew on FFN1, both
+                  operand layouts, the attention projections with Split_K in {1, 2, 4, 7} and
+                  N in {8, 16, 32}, the OPT-66B shapes at N in {8, 16, 32}, the OPT-175B shapes,
+                  the 2:4 + residual split, and the 64-layer decoder stack's time per token step.
+                  The sweep's weights are drawn and encoded on the GPU.
+
+--hetero times the 2:4 + residual path beside the Tiled-CSL path on one weight shape and prints
+one line per sparsity and token count instead of the JSON line.
 
 One GPU only: --gpus above 1 exits with a message.
 """
@@ -45,11 +54,19 @@ HBM_PEAK_GBPS = 8000.0
 # each scaled by what the same counter reads for a copy kernel of known size); summaries of
 # those runs are kept under profiles/.  Keyed by (workload, N, split_k); None where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("opt30b_ffn1", 16, 1): 168.70e6,  # mode 1: no partial sums
-    ("opt30b_ffn1", 16, 8): 175.50e6,  # mode 0: plus 7.34 MB of partial sums
+    # (workload, N, split_k, sparsity): (bytes, profile that holds the counter run)
+    ("opt30b_ffn1", 16, 1, 0.8): (168.70e6, "profiles/tcsl_spmm_kernel_opt30b_ffn1_n16_pmc.txt"),  # mode 1: no partial sums
+    ("opt30b_ffn1", 16, 8, 0.8): (175.50e6, "profiles/tcsl_spmm_kernel_opt30b_ffn1_n16_pmc.txt"),  # mode 0: plus 7.34 MB of partial sums
 }
 TRAFFIC_SOURCE = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, scaled by a copy kernel of known "
-                  "size; summary in profiles/tcsl_spmm_kernel_opt30b_ffn1_n16_pmc.txt (not measured live)")
+                  "size; summary in the named profile (not measured live)")
+
+
+def measured_traffic(workload, N, split_k, sparsity, skew):
+    """(bytes per launch, profile file) from a kept counter run of exactly this case, else (None, None)."""
+    if skew:
+        return None, None
+    return MEASURED_TRAFFIC_BYTES.get((workload, N, split_k, sparsity), (None, None))
 PREWARM_SECONDS = 0.3
 FP16_MFMA_PEAK_TFLOPS = 2500.0
 
@@ -63,6 +80,10 @@ WORKLOADS = {
     "opt66b_outproj": (9216, 9216, 16, 0.8, False),
     "opt66b_ffn1": (36864, 9216, 16, 0.8, False),
     "opt66b_ffn2": (9216, 36864, 16, 0.8, False),
+    "opt175b_qkv": (36864, 12288, 16, 0.8, False),
+    "opt175b_outproj": (12288, 12288, 16, 0.8, False),
+    "opt175b_ffn1": (49152, 12288, 16, 0.8, False),
+    "opt175b_ffn2": (12288, 49152, 16, 0.8, False),
     "config1": (1024, 1024, 8, 0.8, False),
 }
 
@@ -149,48 +170,76 @@ def events_ms(lib, sptr, call, n):
     return ms
 
 
-SWEEP = [
-    # (label, workload, N, sparsity, row_skewed); a label ending in _row_major goes through
-    # SpMM_SplitK_API_RowMajor (B[K][N], C[M][N]: this fork's own operand layout)
-    ("ffn1_n16_row_major", "opt30b_ffn1", 16, 0.8, False),
-    ("ffn1_n64_row_major", "opt30b_ffn1", 64, 0.8, False),
-    ("ffn1_n8", "opt30b_ffn1", 8, 0.8, False),
-    ("ffn1_n32", "opt30b_ffn1", 32, 0.8, False),
-    ("ffn1_n64", "opt30b_ffn1", 64, 0.8, False),
-    ("ffn1_70pct", "opt30b_ffn1", 16, 0.7, False),
-    ("ffn1_90pct", "opt30b_ffn1", 16, 0.9, False),
-    ("ffn1_skewed", "opt30b_ffn1", 16, 0.8, True),
-    ("ffn2", "opt30b_ffn2", 16, 0.8, False),
-    ("qkv", "opt30b_qkv", 16, 0.8, False),
-    ("outproj", "opt30b_outproj", 16, 0.8, False),
-    ("opt66b_qkv", "opt66b_qkv", 16, 0.8, False),
-    ("opt66b_outproj", "opt66b_outproj", 16, 0.8, False),
-    ("opt66b_ffn1", "opt66b_ffn1", 16, 0.8, False),
-    ("opt66b_ffn2", "opt66b_ffn2", 16, 0.8, False),
-]
+def sweep_cases():
+    """(label, workload, N, sparsity, row_skewed, split_k); split_k 0 = the planner's choice for the
+    weight's density.  A label ending in _row_major goes through SpMM_SplitK_API_RowMajor (B[K][N],
+    C[M][N]: this fork's own operand layout).  Cases that share a weight are adjacent."""
+    cases = [
+        ("ffn1_n16_row_major", "opt30b_ffn1", 16, 0.8, False, 0),
+        ("ffn1_n64_row_major", "opt30b_ffn1", 64, 0.8, False, 0),
+        ("ffn1_n8", "opt30b_ffn1", 8, 0.8, False, 0),
+        ("ffn1_n32", "opt30b_ffn1", 32, 0.8, False, 0),
+        ("ffn1_n64", "opt30b_ffn1", 64, 0.8, False, 0),
+        ("ffn1_70pct", "opt30b_ffn1", 16, 0.7, False, 0),
+        ("ffn1_90pct", "opt30b_ffn1", 16, 0.9, False, 0),
+        ("ffn1_skewed", "opt30b_ffn1", 16, 0.8, True, 0),
+        ("ffn2", "opt30b_ffn2", 16, 0.8, False, 0),
+        ("ffn2_n64", "opt30b_ffn2", 64, 0.8, False, 0),
+    ]
+    # the attention projections: the planner's choice and the sweep's Split_K in {1, 2, 4, 7}, N in {8, 16, 32}
+    for name in ("qkv", "outproj"):
+        for N in (16, 8, 32):
+            cases.append((name if N == 16 else f"{name}_n{N}", f"opt30b_{name}", N, 0.8, False, 0))
+            for split_k in (1, 2, 4, 7):
+                cases.append((f"{name}_n{N}_split{split_k}", f"opt30b_{name}", N, 0.8, False, split_k))
+    for model in ("opt66b", "opt175b"):
+        for name in ("qkv", "outproj", "ffn1", "ffn2"):
+            for N in (16, 8, 32):
+                cases.append((f"{model}_{name}" if N == 16 else f"{model}_{name}_n{N}", f"{model}_{name}", N, 0.8, False, 0))
+    return cases
+
+
+def device_weight(G, torch, dev, M, K, sparsity, skew, seed):
+    """A synthetic weight of the benchmark's distribution made and encoded on the GPU (nothing crosses
+    PCIe): N(0, 0.02) fp16 values, kept with probability 1 - sparsity, or, row-skewed, with a per-row
+    probability (1 - sparsity) * Beta(2, 8) / 0.2 (Beta as Gamma(2) / (Gamma(2) + Gamma(8)), a Gamma(k)
+    being minus the log of a product of k uniforms).  Returns (items, offsets) as device tensors; the
+    device encoder gives the bits the host encoder would."""
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    A = torch.randn((M, K), generator=gen, device=dev, dtype=torch.float32)
+    A.mul_(0.02)
+    keep = torch.full((M, 1), 1.0 - sparsity, device=dev)
+    if skew:
+        u = torch.rand((M, 10), generator=gen, device=dev).clamp_min_(1e-12).log_().neg_()
+        x, y = u[:, :2].sum(1, keepdim=True), u[:, 2:].sum(1, keepdim=True)
+        keep = ((1.0 - sparsity) * (x / (x + y)) / 0.2).clamp_max_(1.0)
+    A.mul_(torch.rand((M, K), generator=gen, device=dev) < keep)
+    A = A.to(torch.float16)
+    items, offsets = G.encode_on_device(A)
+    return items, offsets
 
 
 def sweep(G, lib, torch, dev, sptr, with_stack):
-    """The benchmark's other configurations: whole calls (main kernel + reduction) between two
-    events, 300 calls after a pre-warm, weights rotated over > 640 MB of copies."""
+    """The benchmark's other configurations.  Per case: whole calls (main kernel + reduction) between
+    two events, 100 calls after a pre-warm, median of three; the main kernel alone the same way; weights
+    rotated over > 640 MB of copies."""
     out = []
     cache = {}
-    for label, workload, N, sparsity, skew in SWEEP:
+    for label, workload, N, sparsity, skew, forced_split in sweep_cases():
         M, K = WORKLOADS[workload][:2]
         key = (workload, sparsity, skew)
         if key not in cache:
             cache.clear()  # one weight resident at a time
-            A = G.synth_weights(M, K, sparsity, skew, seed=1234)
-            items, offsets = G.InitSparseMatrixA_API(A)
-            del A
-            a_bytes = 16 * int(offsets[-1])
+            torch.cuda.empty_cache()
+            items, offsets = device_weight(G, torch, dev, M, K, sparsity, skew, seed=1234)
+            a_bytes = 4 * items.numel()
             copies = min(64, max(2, -(-640 * 1024 * 1024 // max(a_bytes, 1))))
-            d_items = [torch.from_numpy(items.view(np.int32)).to(dev)]
-            d_items += [d_items[0].clone() for _ in range(copies - 1)]
-            d_offs = [torch.from_numpy(offsets).to(dev) for _ in range(copies)]
+            d_items = [items] + [items.clone() for _ in range(copies - 1)]
+            d_offs = [offsets] + [offsets.clone() for _ in range(copies - 1)]
             cache[key] = (a_bytes, copies, d_items, d_offs)
         a_bytes, copies, d_items, d_offs = cache[key]
-        split_k = G.SpMM_SuggestSplitK_Bytes(M, N, K, a_bytes // 16)
+        split_k = forced_split or G.SpMM_SuggestSplitK_Bytes(M, N, K, a_bytes // 16)
         d_B = torch.from_numpy(G.synth_activations(N, K, seed=4321).view(np.int16)).to(dev)
         d_C = torch.zeros((N, M), dtype=torch.float16, device=dev)
         d_W = torch.zeros((max(split_k, 1), N, M), dtype=torch.float16, device=dev)
@@ -206,16 +255,33 @@ def sweep(G, lib, torch, dev, sptr, with_stack):
             if rc:
                 raise RuntimeError(f"{'SpMM_SplitK_API_RowMajor' if row_major else 'SpMM_SplitK_API'} -> {rc}")
 
+        def kernel(i):
+            rc = lib.SpMM_SplitK_Partials(sptr, p_items[i % copies], p_offs[i % copies], p_B, p_W if split_k > 1 else p_C,
+                                          M, N, K, split_k)
+            if rc:
+                raise RuntimeError(f"SpMM_SplitK_Partials -> {rc}")
+
         prewarm(call, torch, 0.1)
         ms = float(np.median([events_ms(lib, sptr, call, 100) for _ in range(3)])) / 100
+        kernel_ms = None
+        if not row_major:  # (the kernel-alone entry point takes the column-major layout)
+            for i in range(20):
+                kernel(i)
+            kernel_ms = float(np.median([events_ms(lib, sptr, kernel, 100) for _ in range(3)])) / 100
         torch.cuda.synchronize()
         plan = G.SpMM_PlanLaunch(M, N, K, split_k)
+        traffic, traffic_profile = measured_traffic(workload, N, split_k, sparsity, skew)
         out.append({"case": label, "M": M, "K": K, "N": N, "sparsity": sparsity, "row_skewed": skew, "split_k": split_k,
+                    "split_k_from": "sweep" if forced_split else "planner",
                     "layout": "B[K][N], C[M][N]" if row_major else "B[N][K], C[N][M]",
                     "plan": f"mode {plan['mode']}, {plan['waves']} waves", "compressed_bytes": a_bytes,
                     "ms": ms, "frac": a_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                    "kernel_ms": kernel_ms,
+                    "kernel_frac": a_bytes / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS if kernel_ms else None,
+                    "traffic": traffic, "traffic_profile": traffic_profile,
                     "tflops": 2.0 * M * N * K / (ms * 1e-3) / 1e12})
     cache.clear()
+    torch.cuda.empty_cache()
     for sparsity in (0.6, 0.7):
         out.append(split_case(G, lib, torch, dev, sptr, "opt30b_ffn1", 16, sparsity))
     if with_stack:
@@ -371,6 +437,87 @@ def stack_step(G, torch, dev, layers=64, h=9216, N=16, sparsity=0.8, split=False
             "hbm_floor_ms": weight_bytes / (HBM_PEAK_GBPS * 1e9) * 1e3, "build_s": build_s}
 
 
+def hetero_mode(args):
+    """Times the 2:4 + residual path beside the Tiled-CSL path on one weight shape.  For each sparsity
+    the weight is split as the reference's benchmark does (kernel_benchmark/spmm_test.cu:285-330:
+    decompose, then one device form per part) and five figures are printed per token count, in
+    microseconds per call (events around --hetero-iters calls, weights rotated over three copies so
+    that no cache level holds the stream):
+      csl     SpMM_SplitK_API on the whole matrix with the planner's Split_K;
+      a1      the 2:4 kernel alone (its bytes do not depend on the sparsity);
+      hybrid  HeteroSparse_SpMM_API: 2:4 kernel, then the residual's Tiled-CSL kernel, which adds all
+              slabs up itself where its launch allows, else one reduction kernel;
+      2-str   the same with HETERO_FLAG_TWO_STREAMS (the two kernels side by side);
+      fused   HeteroSparse_Fused_SpMM_API: both parts in the 2:4 kernel's launch (residual as lists)."""
+    import torch
+
+    import graphneuralnetproj_amd as G
+
+    G.load_library()
+    M, K = (int(x) for x in args.hetero_shape.lower().split("x"))
+    dev = torch.device("cuda:0")
+    st = torch.cuda.current_stream()
+    iters, c = args.hetero_iters, 3
+
+    def up(a):
+        a = np.ascontiguousarray(a)
+        a = a.view(np.int16) if a.dtype == np.float16 else a.view(np.int32) if a.dtype == np.uint32 else a
+        return torch.from_numpy(a).to(dev) if a.size else torch.zeros(4, dtype=torch.int32, device=dev)
+
+    def time_us(fn):
+        for i in range(iters // 4):
+            fn(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(iters):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters * 1e3
+
+    for sp in [int(x) for x in args.hetero_sparsity.split(",")]:
+        A = G.synth_weights(M, K, sp / 100.0, False, seed=sp)
+        A1, A2 = G.HeteroSparse_Decompose(A)
+        packed = G.HeteroSparse_PackA1(A1)
+        items, offs = G.InitSparseMatrixA_API(A)
+        items2, offs2 = G.InitSparseMatrixA_API(A2)
+        words, woffs, longest = G.HeteroSparse_PackA2(A2)
+        share = float((A2 != 0).sum()) / max(1, int((A != 0).sum()))
+        print(f"# {M}x{K} at {sp} %: Tiled-CSL {items.nbytes / 1e6:.1f} MB; 2:4 records {packed.nbytes / 1e6:.1f} MB + "
+              f"residual {items2.nbytes / 1e6:.1f} MB ({100 * share:.1f} % of the kept values)", flush=True)
+        d_items, d_offs = [up(items) for _ in range(c)], [up(offs) for _ in range(c)]
+        d_p, d_i2, d_o2 = [up(packed) for _ in range(c)], [up(items2) for _ in range(c)], [up(offs2) for _ in range(c)]
+        d_w, d_wo = [up(words) for _ in range(c)], [up(woffs) for _ in range(c)]
+        first = True
+        for N in [int(x) for x in args.hetero_n.split(",")]:
+            B = up(G.synth_activations(N, K, seed=1))
+            C = torch.empty((N, M), dtype=torch.float16, device=dev)
+            s0 = G.SpMM_SuggestSplitK(M, N, K)
+            s1 = G.HeteroSparse_SuggestSplitK(M, N, K)
+            W = torch.empty((s0 + s1 + 64, N, M), dtype=torch.float16, device=dev)
+            if first:  # the host work above let the clocks drop: bring them back before timing anything
+                for i in range(1500):
+                    G.SpMM_SplitK_API(st, None, d_items[i % c], d_offs[i % c], B, C, M, N, K, W, s0)
+                torch.cuda.synchronize()
+                first = False
+            t_csl = time_us(lambda i: G.SpMM_SplitK_API(st, None, d_items[i % c], d_offs[i % c], B, C, M, N, K, W, s0))
+            t_a1 = time_us(lambda i: G.HeteroSparse_A1_Partials(st, d_p[i % c], B, W, M, N, K, s1))
+            S2 = args.hetero_residual_split_k or s0
+            t_h = time_us(lambda i: G.HeteroSparse_SpMM_API(st, d_p[i % c], d_i2[i % c], d_o2[i % c], B, C, M, N, K, W, s1, S2))
+            t_2 = time_us(lambda i: G.HeteroSparse_SpMM_API(st, d_p[i % c], d_i2[i % c], d_o2[i % c], B, C, M, N, K, W, s1, S2,
+                                                           G.HETERO_FLAG_TWO_STREAMS))
+            t_f = float("nan")
+            if longest <= G.HETERO_FUSED_MAX_LIST:
+                t_f = time_us(lambda i: G.HeteroSparse_Fused_SpMM_API(st, d_p[i % c], d_w[i % c], d_wo[i % c], longest, B, C, M, N, K,
+                                                                      W, s1))
+            print(f"sparsity {sp} N={N:2d}: csl {t_csl:6.1f} us (Split_K {s0}) | a1 {t_a1:6.1f} us (Split_K {s1}, "
+                  f"{packed.nbytes / t_a1 / 1e6:.2f} TB/s) | hybrid {t_h:6.1f} us (residual Split_K {S2}) | 2-str {t_2:6.1f} us | "
+                  f"fused {t_f:6.1f} us ({(packed.nbytes + words.nbytes) / t_f / 1e6:.2f} TB/s, longest list {longest})", flush=True)
+        del d_items, d_offs, d_p, d_i2, d_o2, d_w, d_wo
+        torch.cuda.empty_cache()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -395,11 +542,22 @@ def main():
     ap.add_argument("--calibration-copies", type=int, default=0,
                     help="after the timed regions, run this many device-to-device copies of the compressed "
                          "weight (SpMM_CalibrationCopy): a kernel of known traffic for scaling byte counters")
+    ap.add_argument("--hetero", action="store_true",
+                    help="time the 2:4 + residual path beside Tiled-CSL on one shape and print one line per case (no JSON)")
+    ap.add_argument("--hetero-shape", default="28672x7168", help="MxK of --hetero")
+    ap.add_argument("--hetero-sparsity", default="50,60,70,80", help="sparsities of --hetero, in percent")
+    ap.add_argument("--hetero-n", default="8,16,32,64", help="token counts of --hetero")
+    ap.add_argument("--hetero-iters", type=int, default=200)
+    ap.add_argument("--hetero-residual-split-k", type=int, default=0,
+                    help="Split_K of the residual's Tiled-CSL kernel (0 = the planner's choice for the whole matrix)")
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).", file=sys.stderr)
         sys.exit(2)
+    if args.hetero:
+        hetero_mode(args)
+        return
 
     import torch
 
@@ -558,9 +716,9 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": kernel_gbps / HBM_PEAK_GBPS,
-            "traffic": (MEASURED_TRAFFIC_BYTES.get((args.workload, N, split_k))
-                        if sparsity == 0.8 and not skew else None),
+            "traffic": measured_traffic(args.workload, N, split_k, sparsity, skew)[0],
             "traffic_source": TRAFFIC_SOURCE,
+            "traffic_profile": measured_traffic(args.workload, N, split_k, sparsity, skew)[1],
             "kernel": "tcsl_spmm_kernel",
             "kernel_ms_avg": kernel_ms_avg,
             "kernel_launches_timed": kernel_launches,

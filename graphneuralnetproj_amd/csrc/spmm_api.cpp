@@ -445,6 +445,16 @@ extern "C" void SpMM_SynthActivations(uint16_t* B_h, long count, uint64_t seed)
     tcsl::synth_activations(B_h, count, seed);
 }
 
+extern "C" void SpMM_SynthHarnessWeights(uint16_t* A_h, int M, int K, double sparsity, int row_skewed, uint64_t seed)
+{
+    tcsl::synth_harness_weights(A_h, M, K, sparsity, row_skewed, seed);
+}
+
+extern "C" void SpMM_SynthHarnessActivations(uint16_t* B_h, long count, uint64_t seed)
+{
+    tcsl::synth_harness_activations(B_h, count, seed);
+}
+
 extern "C" int SpMM_CalibrationCopy(void* stream, void* dst, const void* src, long bytes)
 {
     if (!dst || !src || bytes < 0 || bytes % 16 != 0)

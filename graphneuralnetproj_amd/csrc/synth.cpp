@@ -13,6 +13,12 @@
 // end2end_inference/ft_tools/huggingface_opt_convert_Phase2.py:68-71) with
 // normally distributed magnitudes instead of its constant 1.0 weights
 // (kernel_benchmark/spmm_test_utils.h:108-141).
+//
+// The harness's own value pattern is there as well (synth_harness_*): every kept
+// weight exactly 1.0 and every activation one of -5, -3, -1, 1, 3
+// (kernel_benchmark/spmm_test_utils.h:111-141), with the keep decisions of the
+// generator above.  Every product and every partial sum is then a small integer,
+// exact in fp32, so a whole output can be checked bit for bit.
 #include <atomic>
 #include <cmath>
 #include <cstdint>
@@ -97,7 +103,34 @@ void for_rows(long rows, F fn)
 
 }  // namespace
 
+namespace {
+void weights(uint16_t* A, int M, int K, double sparsity, int row_skewed, uint64_t seed, bool ones);
+}
+
 void synth_weights(uint16_t* A, int M, int K, double sparsity, int row_skewed, uint64_t seed)
+{
+    weights(A, M, K, sparsity, row_skewed, seed, false);
+}
+
+void synth_harness_weights(uint16_t* A, int M, int K, double sparsity, int row_skewed, uint64_t seed)
+{
+    weights(A, M, K, sparsity, row_skewed, seed, true);
+}
+
+void synth_harness_activations(uint16_t* B, long count, uint64_t seed)
+{
+    // (rand() % 5) / 5 - 0.5) * 10 of the reference: -5, -3, -1, 1, 3 as fp16 bit patterns
+    static const uint16_t kValues[5] = {0xc500, 0xc200, 0xbc00, 0x3c00, 0x4200};
+    const long chunk = 4096;
+    for_rows((count + chunk - 1) / chunk, [&](long c) {
+        const long end = (c + 1) * chunk < count ? (c + 1) * chunk : count;
+        for (long i = c * chunk; i < end; i++)
+            B[i] = kValues[mix(mix(seed ^ (5 * 0xd1342543de82ef95ull)) + static_cast<uint64_t>(i)) % 5];
+    });
+}
+
+namespace {
+void weights(uint16_t* A, int M, int K, double sparsity, int row_skewed, uint64_t seed, bool ones)
 {
     const double keep_mean = 1.0 - sparsity;
     for_rows(M, [&](long m) {
@@ -115,10 +148,11 @@ void synth_weights(uint16_t* A, int M, int K, double sparsity, int row_skewed, u
         uint16_t* row = A + static_cast<size_t>(m) * K;
         for (int k = 0; k < K; k++) {
             const uint64_t idx = static_cast<uint64_t>(m) * static_cast<uint64_t>(K) + k;
-            row[k] = unit(seed, 1, idx) < p ? to_half(0.02f * normal(seed, 2, idx)) : 0;
+            row[k] = unit(seed, 1, idx) < p ? (ones ? uint16_t(0x3c00) : to_half(0.02f * normal(seed, 2, idx))) : 0;
         }
     });
 }
+}  // namespace
 
 void synth_activations(uint16_t* B, long count, uint64_t seed)
 {

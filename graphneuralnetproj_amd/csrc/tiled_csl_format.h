@@ -34,5 +34,8 @@ int encode_file(const char* dense, int M, int K, const char* nz_path, const char
 // Deterministic synthetic inputs (counter based, identical on every host).
 void synth_weights(uint16_t* A, int M, int K, double sparsity, int row_skewed, uint64_t seed);
 void synth_activations(uint16_t* B, long count, uint64_t seed);
+// The same keep decisions with the value pattern of the reference's harness: weights 1.0, activations in {-5, -3, -1, 1, 3}.
+void synth_harness_weights(uint16_t* A, int M, int K, double sparsity, int row_skewed, uint64_t seed);
+void synth_harness_activations(uint16_t* B, long count, uint64_t seed);
 
 }  // namespace tcsl

@@ -152,6 +152,10 @@ def load_library():
                                       ctypes.c_uint64]
     lib.SpMM_SynthActivations.restype = None
     lib.SpMM_SynthActivations.argtypes = [_u16p, ctypes.c_long, ctypes.c_uint64]
+    lib.SpMM_SynthHarnessWeights.restype = None
+    lib.SpMM_SynthHarnessWeights.argtypes = lib.SpMM_SynthWeights.argtypes
+    lib.SpMM_SynthHarnessActivations.restype = None
+    lib.SpMM_SynthHarnessActivations.argtypes = lib.SpMM_SynthActivations.argtypes
     lib.SpMM_CalibrationCopy.restype = ctypes.c_int
     lib.SpMM_CalibrationCopy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_long]
     lib.SpMM_SplitK_API_Events.restype = ctypes.c_int
@@ -412,6 +416,22 @@ def synth_activations(N, K, seed=0):
     """Deterministic synthetic fp16 activations, one K vector per token (N x K)."""
     B = np.empty((N, K), dtype=np.uint16)
     load_library().SpMM_SynthActivations(B.ctypes.data_as(_u16p), N * K, seed)
+    return B.view(np.float16)
+
+
+def synth_harness_weights(M, K, sparsity, row_skewed=False, seed=0):
+    """The reference harness's weights (kernel_benchmark/spmm_test_utils.h:111-123): kept values are
+    exactly 1.0; the keep decisions are those of synth_weights with the same arguments."""
+    A = np.empty((M, K), dtype=np.uint16)
+    load_library().SpMM_SynthHarnessWeights(A.ctypes.data_as(_u16p), M, K, float(sparsity), int(bool(row_skewed)), seed)
+    return A.view(np.float16)
+
+
+def synth_harness_activations(N, K, seed=0):
+    """The reference harness's activations (kernel_benchmark/spmm_test_utils.h:137-141): values in
+    {-5, -3, -1, 1, 3}, one K vector per token (N x K)."""
+    B = np.empty((N, K), dtype=np.uint16)
+    load_library().SpMM_SynthHarnessActivations(B.ctypes.data_as(_u16p), N * K, seed)
     return B.view(np.float16)
 
 

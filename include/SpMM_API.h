@@ -286,6 +286,16 @@ SPMM_EXPORT int SpMM_SplitK_API_Planned(void* stream, const void* Compressed_A, 
  */
 SPMM_EXPORT void SpMM_SynthWeights(uint16_t* A_h, int M, int K, double sparsity, int row_skewed, uint64_t seed);
 SPMM_EXPORT void SpMM_SynthActivations(uint16_t* B_h, long count, uint64_t seed);
+/*
+ * The value pattern of the reference's own harness, init_host_matrices
+ * (kernel_benchmark/spmm_test_utils.h:111-141): every kept weight is exactly 1.0 and every
+ * activation one of -5, -3, -1, 1, 3, here with the seeded keep decisions of SpMM_SynthWeights
+ * (a weight drawn with the same arguments has its non-zeros in the same places) instead of rand().
+ * All products and partial sums are small integers, exact in fp32: the whole output of a product
+ * can be compared bit for bit.
+ */
+SPMM_EXPORT void SpMM_SynthHarnessWeights(uint16_t* A_h, int M, int K, double sparsity, int row_skewed, uint64_t seed);
+SPMM_EXPORT void SpMM_SynthHarnessActivations(uint16_t* B_h, long count, uint64_t seed);
 
 /*
  * Device-to-device streaming copy of `bytes` (multiple of 16) on `stream`; a

@@ -3,8 +3,10 @@ own launch plan: the attention projections with every Split_K of the sweep, the 
 matrices at 70 / 90 % and row-skewed sparsity for 8 to 64 tokens, and the 64-layer decoder stack.
 
 A full CPU product of these sizes takes minutes, so each case checks
-  * sampled output rows against the oracle's fp32 product (|gpu - ref| <= 1e-2 + 1e-2 |ref|), and
+  * sampled output rows against the oracle's fp32 product (|gpu - ref| <= 1e-2 + 1e-2 |ref|): the
+    first and last rows of the emptiest, the fullest, the first and the last tile row, and random ones, and
   * every row through a property that needs no reference: linearity in the activations.
+Every element of the same shapes is compared bit for bit, on integer-valued data, in test_gpu_exact.py.
 """
 import numpy as np
 import pytest
@@ -28,6 +30,17 @@ def _close(C, ref):
     err = np.abs(C - ref)
     bad = err > ATOL + RTOL * np.abs(ref)
     assert not bad.any(), f"{bad.sum()} elements out of tolerance, max err {err.max()}"
+
+
+def _rows_to_check(offsets, M, K, seed, random_rows=64):
+    """Rows for the comparison with the oracle: every row of the emptiest and of the fullest tile
+    row's first and last 16 (where the kernel changes its segment length, clears whole tiles or
+    lets more waves stream), plus random ones."""
+    per_tile_row = np.diff(offsets[:-1].astype(np.int64)[::K // 64])
+    picks = {int(per_tile_row.argmin()), int(per_tile_row.argmax()), 0, M // 128 - 1}
+    rows = [np.arange(128 * t, 128 * t + 16) for t in picks] + [np.arange(128 * t + 112, 128 * t + 128) for t in picks]
+    rows.append(np.random.default_rng(seed).choice(M, size=random_rows, replace=False))
+    return np.unique(np.concatenate(rows))
 
 
 def _sampled_rows_and_linearity(spmm, oracle, torch, A, d_items, d_offs, M, K, N, split_k, rows, what):
@@ -60,16 +73,16 @@ def test_attention_projections_every_split(spmm, oracle, M, K):
     items, offsets = spmm.InitSparseMatrixA_API(A)
     d_items = torch.from_numpy(items.view(np.int32)).to(dev)
     d_offs = torch.from_numpy(offsets).to(dev)
-    rows = np.sort(np.random.default_rng(M + K).choice(M, size=96, replace=False))
+    rows = _rows_to_check(offsets, M, K, M + K)
     for N in (8, 16, 32):
         for split_k in (1, 2, 4, 7):
             _sampled_rows_and_linearity(spmm, oracle, torch, A, d_items, d_offs, M, K, N, split_k, rows, "attention projection")
 
 
-@pytest.mark.parametrize("sparsity,skew", [(0.7, False), (0.9, False), (0.8, True)])
+@pytest.mark.parametrize("sparsity,skew", [(0.7, False), (0.9, False), (0.8, True), (0.7, True), (0.9, True), (0.8, False)])
 @pytest.mark.parametrize("M,K", [(28672, 7168), (7168, 28672)])
 def test_feed_forward_sparsity_sweep(spmm, oracle, M, K, sparsity, skew):
-    """OPT-30B FFN1 and FFN2 at 70 % and 90 % Bernoulli and 80 % Beta(2,8) row-skewed sparsity,
+    """OPT-30B FFN1 and FFN2 at 70 / 80 / 90 % sparsity, Bernoulli and Beta(2,8) row-skewed,
     N in {8, 16, 32, 64}, with the planner's Split_K."""
     torch = _torch()
     dev = torch.device("cuda:0")
@@ -80,7 +93,7 @@ def test_feed_forward_sparsity_sweep(spmm, oracle, M, K, sparsity, skew):
         assert per_row.max() > 4 * max(int(per_row.min()), 1)
     d_items = torch.from_numpy(items.view(np.int32)).to(dev)
     d_offs = torch.from_numpy(offsets).to(dev)
-    rows = np.sort(np.random.default_rng(M + K).choice(M, size=96, replace=False))
+    rows = _rows_to_check(offsets, M, K, M + K)
     for N in (8, 16, 32, 64):
         split_k = spmm.SpMM_SuggestSplitK_Bytes(M, N, K, int(offsets[-1]))
         _sampled_rows_and_linearity(spmm, oracle, torch, A, d_items, d_offs, M, K, N, split_k, rows,
@@ -98,7 +111,7 @@ def test_row_major_entry_full_size(spmm, oracle, M, K, sparsity):
     items, offsets = spmm.InitSparseMatrixA_API(A)
     d_items = torch.from_numpy(items.view(np.int32)).to(dev)
     d_offs = torch.from_numpy(offsets).to(dev)
-    rows = np.sort(np.random.default_rng(M + K).choice(M, size=96, replace=False))
+    rows = _rows_to_check(offsets, M, K, M + K)
     for N in (8, 16, 32, 64):
         split_k = spmm.SpMM_SuggestSplitK_Bytes(M, N, K, int(offsets[-1]))
         B = spmm.synth_activations(N, K, seed=9 + N)

@@ -114,6 +114,41 @@ def test_dense_tile_closed_form(oracle):
     assert np.array_equal(items, want.reshape(-1))
 
 
+@pytest.mark.parametrize("extra", [4, 8])
+def test_full_round_plus_tail_hand_derived(oracle, spmm, extra):
+    """A tile with one full round of 32 vectors AND a tail (R = 1, Rem = 1 or 2), worked out by hand
+    from csrc/SpMM_API.cu:379-424.  Rows 0 and 8 are full (row % 8 == 0: no swizzle, column n sits in
+    bank n / 2), so every bank stacks [r0 c2b, r0 c2b+1, r8 c2b, r8 c2b+1]; row 16 adds columns
+    0 .. extra-1, two more words on top of banks 0 .. extra/2-1.  No padding (132 or 136 words).
+      Tail first (:384-391), v outer, b inner, always the fullest stack, lowest bank on ties:
+        extra = 4: b0 b1 b0 b1 give (16,1) (16,3) (16,0) (16,2), all to Tail[0];
+        extra = 8: b0 b1 b2 b3 b0 b1 b2 b3 give (16,1) (16,3) (16,5) (16,7) (16,0) (16,2) (16,4) (16,6),
+                   dealt alternately to Tail[0] and Tail[1].
+      Then the round (:394-403): all stacks hold 4, so each of its four passes pops banks 0 .. 31 in
+      order and Main[b] = bank b's words from the top down.
+      Emitted last in, first out (:406-424): vector b of the round = bank b's words in scan order,
+      tail vector b = Tail[b] reversed.
+    Drawing the round before the tail, popping first in first out, or breaking ties upwards each
+    gives another order."""
+    A = np.zeros((128, 64), dtype=np.uint16)
+    value = lambda m, n: 0x3C00 + m * 64 + n + 1  # distinct, non-zero, finite
+    for m, cols in ((0, 64), (8, 64), (16, extra)):
+        for n in range(cols):
+            A[m, n] = value(m, n)
+    word = lambda m, n: value(m, n) | ((m * 64 + n) << 16)  # rows 0, 8, 16: position = m * 64 + n
+    want = []
+    for b in range(32):
+        want += [word(0, 2 * b), word(0, 2 * b + 1), word(8, 2 * b), word(8, 2 * b + 1)]
+    if extra == 4:
+        want += [word(16, 2), word(16, 0), word(16, 3), word(16, 1)]
+    else:
+        want += [word(16, 4), word(16, 0), word(16, 5), word(16, 1), word(16, 6), word(16, 2), word(16, 7), word(16, 3)]
+    for encode in (oracle.encode, spmm.InitSparseMatrixA_API):
+        items, offs = encode(A.view(np.float16) if encode is spmm.InitSparseMatrixA_API else A)
+        assert offs.tolist() == [0, len(want) // 4, len(want) // 4]
+        assert items.tolist() == want
+
+
 def test_encode_rejects_bad_shapes(oracle):
     for M, K in [(100, 64), (128, 96), (64, 64), (128, 32)]:
         with pytest.raises(ValueError):
