@@ -46,6 +46,8 @@ EXPORTED_SYMBOLS = (
     "SpMM_DeviceEncodeItems",
     "SpMM_SynthWeights",
     "SpMM_SynthActivations",
+    "SpMM_SynthHarnessWeights",
+    "SpMM_SynthHarnessActivations",
     "SpMM_CalibrationCopy",
     "SpMM_SplitK_API_Events",
     "SpMM_SplitK_Partials",
