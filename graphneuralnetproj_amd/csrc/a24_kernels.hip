@@ -249,7 +249,16 @@ constexpr int kRowBytes = 272;
 // everything else, so that every unit issues the same number of loads.
 constexpr int kImageBytes = 4096;
 
-template<int NT, int RB, int W, int RL>
+// RM: the operands are row-major, this fork's own layout (csrc/SpMM_Kernel.cuh:372-374 for B,
+// :731-734 for the output): B[k][n] (K x n_tokens, dense), out / fused_out and the slabs [m][n]
+// (M x n_tokens, dense; ldb, ldo and ldc are not used).  A unit's 128 x n_tokens activation block is
+// then one contiguous run: it is staged in LDS as it sits in memory (with 64 tokens the four
+// 32-byte column chunks of a row are permuted by (k >> 1) & 3, so that the four rows one read touches
+// fall into different banks) and read back with the transposing LDS read ds_read_b64_tr_b16, which
+// hands lane i of a group of sixteen the i-th column of a 4 x 16 block whose rows the sixteen lanes
+// address four to a row: two such reads give a lane the eight consecutive k of its token that the
+// matrix instructions want.
+template<int NT, int RB, int W, int RL, bool RM = false>
 __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8_t* __restrict__ packed,
                                                                      const _Float16* __restrict__ B,
                                                                      _Float16* __restrict__ out, int units,
@@ -277,14 +286,27 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
     for (int r = 0; r < RB; r++)
         rec[r] = block_records(packed, block0 + r, units);
     // this thread's chunks of the activation tile: token c / 16, columns (c % 16) * 8 .. + 8
+    // (RM: chunk c of the unit's contiguous block, i.e. tokens 8 (c % (n_tokens / 8)) .. + 7 of row
+    // c / (n_tokens / 8), kept where it sits in memory)
+    auto rm_byte = [&](int k, int n) {  // LDS byte of B[unit's row k][token n], RM only
+        return n_tokens == 64 ? k * 128 + ((((n >> 4) ^ (k >> 1)) & 3) << 5) + (n & 15) * 2 : (k * n_tokens + n) * 2;
+    };
     const _Float16* src[CH];
     int dst[CH];
+    const size_t unit_step = RM ? (size_t)128 * n_tokens : 128;  // elements between a chunk's places in two consecutive units
 #pragma unroll
     for (int i = 0; i < CH; i++) {
         const int c = tid + i * kThreads;
-        const int n = c < n_tokens * 16 ? c >> 4 : 0;
-        src[i] = B + (size_t)n * ldb + (c & 15) * 8;
-        dst[i] = n * kRowBytes + (c & 15) * 16;
+        if constexpr (RM) {
+            const int cc = c < n_tokens * 16 ? c : 0;
+            const int per_row_log2 = __builtin_ctz(n_tokens >> 3);
+            src[i] = B + (size_t)cc * 8;
+            dst[i] = rm_byte(cc >> per_row_log2, 8 * (cc & ((1 << per_row_log2) - 1)));
+        } else {
+            const int n = c < n_tokens * 16 ? c >> 4 : 0;
+            src[i] = B + (size_t)n * ldb + (c & 15) * 8;
+            dst[i] = n * kRowBytes + (c & 15) * 16;
+        }
     }
     // where this lane's fragments sit in a buffer (with more than 16 tokens every token block is
     // full, so the blocks are a constant apart: one register instead of NT)
@@ -296,6 +318,24 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
             n = n < n_tokens ? n : n_tokens - 1;
         frag[t] = n * kRowBytes + (lane >> 4) * 16;
     }
+    // RM: where the two transposing reads (hh = 0, 1) of step 0 for token block t start: lane j of a
+    // group of sixteen points at row 8 (lane / 16) + 4 hh + j / 4, tokens 16 t + 4 (j % 4) .. + 3 (with
+    // 8 tokens the upper half repeats the lower); a step further is 32 rows further.  Everything
+    // but the lane's own part is a constant of (t, hh): with 64 tokens the permuted chunk is
+    // t ^ (2 hh + j / 8), whose bit 1 is constant and whose bit 0 is j / 8 for even t and its
+    // complement for odd t, so two registers serve all blocks.
+    int tr_lane[2] = {0, 0};
+    const int rm_row_bytes = NT == 4 ? 128 : 2 * n_tokens;
+    if constexpr (RM) {
+        const int l15 = lane & 15;
+        const int base0 = (8 * (lane >> 4) + (l15 >> 2)) * rm_row_bytes + ((4 * (l15 & 3)) & (n_tokens - 1)) * 2;
+        tr_lane[0] = NT == 4 ? base0 + 32 * (l15 >> 3) : base0;
+        tr_lane[1] = NT == 4 ? base0 + 32 - 32 * (l15 >> 3) : base0;
+    }
+    auto tr_at = [&](int t, int hh) {
+        return NT == 4 ? tr_lane[t & 1] + 512 * hh + 64 * ((t >> 1) ^ hh) : tr_lane[0] + 4 * hh * rm_row_bytes + 32 * t;
+    };
+    const int tr_step = 32 * rm_row_bytes;
 
     // The residual's dense products get accumulators of their own, added to the others at the end:
     // a dense MFMA that takes the sparse instruction's result as its addend directly behind it read
@@ -335,7 +375,7 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
             asm volatile("global_load_dword %0, %1, off" : "=v"(x.next) : "v"(off_lane + (size_t)unit_after * kGroupBlocks));
 #pragma unroll
         for (int i = 0; i < CH; i++)
-            x.stage[i] = issue_b(src[i] + (size_t)unit * 128);
+            x.stage[i] = issue_b(src[i] + (size_t)unit * unit_step);
 #pragma unroll
         for (int r = 0; r < RB; r++)
             x.a[r] = issue_a(rec[r] + (size_t)unit * kUnitStride + lane * 16, rec[r] + (size_t)unit * kUnitStride + lane * 4);
@@ -419,8 +459,20 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
         for (int t = 0; t < NT; t++) {
             half8 f[4];
 #pragma unroll
-            for (int s = 0; s < 4; s++)
-                f[s] = *reinterpret_cast<const half8*>(tile + buf * kBuf + frag[t] + s * 64);
+            for (int s = 0; s < 4; s++) {
+                if constexpr (RM) {
+                    typedef short short4v __attribute__((ext_vector_type(4)));
+                    typedef short short8v __attribute__((ext_vector_type(8)));
+                    typedef __attribute__((address_space(3))) short4v lds_short4v;
+                    const unsigned char* const at = tile + buf * kBuf + s * tr_step;
+                    const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v*)(at + tr_at(t, 0)));
+                    const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v*)(at + tr_at(t, 1)));
+                    const short8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    f[s] = __builtin_bit_cast(half8, both);
+                } else {
+                    f[s] = *reinterpret_cast<const half8*>(tile + buf * kBuf + frag[t] + s * 64);
+                }
+            }
 #pragma unroll
             for (int r = 0; r < RB; r++) {
                 acc[r][t] = __builtin_amdgcn_smfmac_f32_16x16x32_f16(step_values(a[r], 0), f[0], acc[r][t], (int)a[r].idx, 0, 0);
@@ -541,11 +593,22 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
                     s = float4v{fmaxf(s[0], 0.f), fmaxf(s[1], 0.f), fmaxf(s[2], 0.f), fmaxf(s[3], 0.f)};
                 half4 h = {static_cast<_Float16>(s[0]), static_cast<_Float16>(s[1]), static_cast<_Float16>(s[2]),
                            static_cast<_Float16>(s[3])};
-                _Float16* const to = dstc + (size_t)n * ldo + (block0 + r) * 16 + (lane >> 4) * 4;
-                if (arrivals)
-                    inlaunch::store_through(to, h);
-                else
-                    *reinterpret_cast<half4*>(to) = h;
+                if constexpr (RM) {  // [m][n]: the sixteen tokens of a row are adjacent (sixteen lanes to a 32-byte segment)
+                    _Float16* const to = dstc + ((size_t)(block0 + r) * 16 + (lane >> 4) * 4) * n_tokens + n;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        if (arrivals)
+                            inlaunch::store_through(to + (size_t)i * n_tokens, h[i]);
+                        else
+                            to[(size_t)i * n_tokens] = h[i];
+                    }
+                } else {
+                    _Float16* const to = dstc + (size_t)n * ldo + (block0 + r) * 16 + (lane >> 4) * 4;
+                    if (arrivals)
+                        inlaunch::store_through(to, h);
+                    else
+                        *reinterpret_cast<half4*>(to) = h;
+                }
             }
         }
     }
@@ -556,10 +619,10 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
     if (arrivals)
         inlaunch::fused_reduction_tail(out, fused_out, M, n_tokens, static_cast<int>(ldc), gridDim.y, relu,
                                        blockIdx.x * (16 * RB * W), 16 * RB * W, arrivals + blockIdx.x,
-                                       reinterpret_cast<unsigned int*>(tile), W * kWave, false);
+                                       reinterpret_cast<unsigned int*>(tile), W * kWave, RM);
 }
 
-template<int NT, int RB, int W, int RL>
+template<int NT, int RB, int W, int RL, bool RM>
 int launch_shared_b(hipStream_t stream, const void* packed, const void* B, void* out, int M, int N, int K, int split_k,
                     long ldb, long ldo, long slab, const void* words, const void* offsets, int relu, void* fused_out,
                     unsigned int* arrivals, long ldc)
@@ -569,7 +632,7 @@ int launch_shared_b(hipStream_t stream, const void* packed, const void* B, void*
     if (M % (16 * RB * W) != 0)
         return static_cast<int>(hipErrorInvalidValue);
     const unsigned lds = 2 * NT * 16 * kRowBytes + (RL > 0 ? W * kImageBytes : 0);
-    auto kern = a24_spmm_shared_b_kernel<NT, RB, W, RL>;
+    auto kern = a24_spmm_shared_b_kernel<NT, RB, W, RL, RM>;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess)
@@ -587,20 +650,32 @@ int launch_shared_b(hipStream_t stream, const void* packed, const void* B, void*
 template<int NT>
 int launch_shared_b_nt(hipStream_t s, const void* packed, const void* B, void* out, int M, int N, int K, int split_k, int rb,
                        int waves, long ldb, long ldo, long slab, int rl, const void* words, const void* offsets, int relu,
-                       void* fused_out, unsigned int* arrivals, long ldc)
+                       void* fused_out, unsigned int* arrivals, long ldc, bool row_major)
 {
+#define A24_GO(RB_, W_, RL_, RM_) \
+    launch_shared_b<NT, RB_, W_, RL_, RM_>(s, packed, B, out, M, N, K, split_k, ldb, ldo, slab, words, offsets, relu, fused_out, arrivals, ldc)
+    // the library's own launch shapes (two row blocks per wave) take either operand layout
 #define A24_CASE(RB_, W_, RL_)                   \
     if (rb == RB_ && waves == W_ && rl == RL_) \
-        return launch_shared_b<NT, RB_, W_, RL_>(s, packed, B, out, M, N, K, split_k, ldb, ldo, slab, words, offsets, relu, \
-                                                 fused_out, arrivals, ldc);
+        return row_major ? A24_GO(RB_, W_, RL_, true) : A24_GO(RB_, W_, RL_, false);
+#define A24_CASE_COLUMN_MAJOR(RB_, W_, RL_)                     \
+    if (rb == RB_ && waves == W_ && rl == RL_ && !row_major) \
+        return A24_GO(RB_, W_, RL_, false);
     A24_CASE(2, 4, 0) A24_CASE(2, 8, 0)
     A24_CASE(2, 4, 1) A24_CASE(2, 8, 1) A24_CASE(2, 4, 2) A24_CASE(2, 8, 2) A24_CASE(2, 4, 3) A24_CASE(2, 8, 3)
-    A24_CASE(2, 4, 4) A24_CASE(2, 4, 5) A24_CASE(2, 8, 4)
-    if constexpr (NT <= 2) {
-        A24_CASE(2, 8, 5)  // with 64 tokens it would not fit 256 registers  // three record sets of four row blocks do not fit the registers beside 64 tokens
-        A24_CASE(4, 2, 0) A24_CASE(4, 4, 0) A24_CASE(4, 8, 0)
+    A24_CASE(2, 4, 4) A24_CASE(2, 4, 5)
+    if constexpr (NT > 2) {
+        A24_CASE_COLUMN_MAJOR(2, 8, 4)  // (row-major with 64 tokens: one register too many for eight waves)
     }
+    if constexpr (NT <= 2) {
+        A24_CASE(2, 8, 4)
+        A24_CASE(2, 8, 5)  // with 64 tokens it would not fit 256 registers
+        // (three record sets of four row blocks do not fit the registers beside 64 tokens)
+        A24_CASE_COLUMN_MAJOR(4, 2, 0) A24_CASE_COLUMN_MAJOR(4, 4, 0) A24_CASE_COLUMN_MAJOR(4, 8, 0)
+    }
+#undef A24_CASE_COLUMN_MAJOR
 #undef A24_CASE
+#undef A24_GO
     return static_cast<int>(hipErrorInvalidValue);
 }
 
@@ -647,15 +722,17 @@ int launch_nt(hipStream_t s, const void* packed, const void* B, void* out, int M
 // results are written as zero (for a launch that writes the finished result).
 // fuse_page >= 0 (share_b, split_k > 1, ldo == M, slab == M * N): the launch adds its slabs up into
 // fused_out (token stride ldc) itself, counting arrivals on that page of the library's counters.
+// row_major (share_b with rb == 2 only): B is [K][N] and out, the slabs and fused_out [M][N], all
+// dense (ldb, ldo and ldc are not used; slab == M * N).
 extern "C" int a24_launch_spmm(void* stream, const void* packed, const void* B, void* out, int M, int N, int K,
                                int split_k, int rb, int waves, int share_b, long ldb, long ldo, long slab,
                                int residual_loads, const void* words, const void* offsets, int relu, int fuse_page,
-                               void* fused_out, long ldc)
+                               void* fused_out, long ldc, int row_major)
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
     unsigned int* arrivals = nullptr;
     if (fuse_page >= 0) {
-        if (!share_b || split_k < 2 || !fused_out || ldo != M || slab != static_cast<long>(M) * N || rb < 1 || waves < 1
+        if (!share_b || split_k < 2 || !fused_out || (ldo != M && !row_major) || slab != static_cast<long>(M) * N || rb < 1 || waves < 1
             || M / (16 * rb * waves) > 4096 || M % 8 != 0)
             return static_cast<int>(hipErrorInvalidValue);
         if (const int rc = tcsl_counter_page_address(fuse_page, &arrivals))
@@ -665,15 +742,15 @@ extern "C" int a24_launch_spmm(void* stream, const void* packed, const void* B, 
         switch (N) {
             case 8:
             case 16: return launch_shared_b_nt<1>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets, relu,
-                                                     fused_out, arrivals, ldc);
+                                                     fused_out, arrivals, ldc, row_major != 0);
             case 32: return launch_shared_b_nt<2>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets, relu,
-                                                     fused_out, arrivals, ldc);
+                                                     fused_out, arrivals, ldc, row_major != 0);
             case 64: return launch_shared_b_nt<4>(s, packed, B, out, M, N, K, split_k, rb, waves, ldb, ldo, slab, residual_loads, words, offsets, relu,
-                                                     fused_out, arrivals, ldc);
+                                                     fused_out, arrivals, ldc, row_major != 0);
             default: return static_cast<int>(hipErrorInvalidValue);
         }
     }
-    if (residual_loads != 0 || relu)
+    if (residual_loads != 0 || relu || row_major)
         return static_cast<int>(hipErrorInvalidValue);
     switch (N) {
         case 8:

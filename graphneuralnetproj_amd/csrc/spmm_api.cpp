@@ -24,7 +24,7 @@ int tcsl_launch_encode_items(void* stream, const void* A, int M, int K, const in
 int a24_launch_spmm(void* stream, const void* packed, const void* B, void* out, int M, int N, int K, int split_k, int rb,
                     int waves, int share_b, long ldb, long ldo, long slab, int residual_loads = 0,
                     const void* words = nullptr, const void* offsets = nullptr, int relu = 0, int fuse_page = -1,
-                    void* fused_out = nullptr, long ldc = 0);
+                    void* fused_out = nullptr, long ldc = 0, int row_major = 0);
 int a24_launch_split_pack(void* stream, const void* A, void* packed, void* residual, int M, int K);
 int a24_launch_residual_offsets(void* stream, const void* A2, int M, int K, int* offsets, int* longest);
 int a24_launch_residual_words(void* stream, const void* A2, int M, int K, const int* offsets, void* words);
@@ -577,7 +577,10 @@ bool a24_shape_ok(int M, int N, int K, int split_k, int row_blocks, int waves, i
 namespace {
 int a24_split_call(void* stream, const void* Packed_A1, const void* B, long ldb, void* C, long ldc, int M, int N, int K,
                    void* Reduction_Workspace, int Split_K, int row_blocks, int waves, int loads, const void* words,
-                   const void* offsets, int relu, bool separate_reduction);
+                   const void* offsets, int relu, bool separate_reduction, bool row_major = false);
+int hybrid_call(const char* who, void* stream, const void* Packed_A1, const void* Compressed_A2, const int* TileOffsets_A2,
+                const void* B, void* C, int M, int N, int K, void* Reduction_Workspace, int Split_K_A1, int Split_K_A2,
+                int Flags, bool row_major);
 }
 
 extern "C" int HeteroSparse_A1_Partials(void* stream, const void* Packed_A1, const void* B, void* Partials, int M, int N,
@@ -610,6 +613,24 @@ extern "C" int HeteroSparse_SpMM_API(void* stream, const void* Packed_A1, const 
                                      const int* TileOffsets_A2, const void* B, void* C, int M, int N, int K,
                                      void* Reduction_Workspace, int Split_K_A1, int Split_K_A2, int Flags)
 {
+    return hybrid_call("HeteroSparse_SpMM_API", stream, Packed_A1, Compressed_A2, TileOffsets_A2, B, C, M, N, K,
+                       Reduction_Workspace, Split_K_A1, Split_K_A2, Flags, false);
+}
+
+extern "C" int HeteroSparse_SpMM_API_RowMajor(void* stream, const void* Packed_A1, const void* Compressed_A2,
+                                              const int* TileOffsets_A2, const void* B, void* C, int M, int N, int K,
+                                              void* Reduction_Workspace, int Split_K_A1, int Split_K_A2, int Flags)
+{
+    return hybrid_call("HeteroSparse_SpMM_API_RowMajor", stream, Packed_A1, Compressed_A2, TileOffsets_A2, B, C, M, N, K,
+                       Reduction_Workspace, Split_K_A1, Split_K_A2, Flags, true);
+}
+
+namespace {
+// row_major: B is [K][N], C and every slab [M][N] (this fork's layout) instead of [N][K] and [N][M].
+int hybrid_call(const char* who, void* stream, const void* Packed_A1, const void* Compressed_A2, const int* TileOffsets_A2,
+                const void* B, void* C, int M, int N, int K, void* Reduction_Workspace, int Split_K_A1, int Split_K_A2,
+                int Flags, bool row_major)
+{
     const bool residual = Compressed_A2 != nullptr;
     if (N != 8 && N != 16 && N != 32 && N != 64) {
         std::printf("MM_Sparse_API Error: Unsupported N dimension %d!\n", N);  // csrc/SpMM_API.cu:192-193
@@ -621,19 +642,22 @@ extern "C" int HeteroSparse_SpMM_API(void* stream, const void* Packed_A1, const 
     if (!Packed_A1 || !B || !C || (residual && !TileOffsets_A2) || !a24_shape_ok(M, N, K, Split_K_A1, d.row_blocks, d.waves, d.share_b)
         || (residual && (Split_K_A2 < 1 || Split_K_A2 > 65535)) || ((residual || Split_K_A1 > 1) && !Reduction_Workspace)
         || (Flags & ~HETERO_FLAG_TWO_STREAMS)) {
-        std::fprintf(stderr, "HeteroSparse_SpMM_API: unsupported call M=%d N=%d K=%d Split_K=%d/%d (need M %% 128 == 0, K %% 128 == 0, no empty batch, non-null pointers)\n",
-                     M, N, K, Split_K_A1, Split_K_A2);
+        std::fprintf(stderr, "%s: unsupported call M=%d N=%d K=%d Split_K=%d/%d (need M %% 128 == 0, K %% 128 == 0, no empty batch, non-null pointers)\n",
+                     who, M, N, K, Split_K_A1, Split_K_A2);
         return tcsl_error_invalid_value();
     }
+    if (row_major && !d.share_b)  // (the library's plans all share the activation tile; the other kernel takes column-major only)
+        return tcsl_error_invalid_value();
     const long mn = static_cast<long>(M) * N;
     if (!residual && Split_K_A1 == 1)  // the 2:4 kernel writes C itself
-        return a24_launch_spmm(stream, Packed_A1, B, C, M, N, K, 1, d.row_blocks, d.waves, d.share_b, K, M, mn);
+        return a24_launch_spmm(stream, Packed_A1, B, C, M, N, K, 1, d.row_blocks, d.waves, d.share_b, K, M, mn, 0, nullptr, nullptr, 0,
+                               -1, nullptr, 0, row_major ? 1 : 0);
     int rc = 0;
     uint16_t* ws = static_cast<uint16_t*>(Reduction_Workspace);
     if (!residual) {
         if (d.share_b)
             return a24_split_call(stream, Packed_A1, B, K, C, M, M, N, K, ws, Split_K_A1, d.row_blocks, d.waves, 0, nullptr, nullptr,
-                                  0, false);
+                                  0, false, row_major);
         rc = a24_launch_spmm(stream, Packed_A1, B, ws, M, N, K, Split_K_A1, d.row_blocks, d.waves, d.share_b, K, M, mn);
         return rc != 0 ? rc : tcsl_launch_reduce(stream, C, ws, mn, 1, mn, Split_K_A1, 0);
     }
@@ -649,11 +673,12 @@ extern "C" int HeteroSparse_SpMM_API(void* stream, const void* Packed_A1, const 
             return rc;
         CallOptions o;
         o.separate_reduction = true;
+        o.row_major = row_major;
         rc = launch_main(side, Compressed_A2, TileOffsets_A2, B, ws, M, N, K, Split_K_A2, o, K, M, false, nullptr, 0,
                          nullptr);
         if (rc == 0)
             rc = a24_launch_spmm(stream, Packed_A1, B, ws_a1, M, N, K, Split_K_A1, d.row_blocks, d.waves, d.share_b, K, M,
-                                 mn);
+                                 mn, 0, nullptr, nullptr, 0, -1, nullptr, 0, row_major ? 1 : 0);
         // the side stream joins the caller's whatever happened in between: a fork left open would
         // leave the two streams unordered (and invalidate a graph capture that includes this call)
         const int joined = a24_side_end(stream, side);
@@ -664,9 +689,10 @@ extern "C" int HeteroSparse_SpMM_API(void* stream, const void* Packed_A1, const 
         // its launch shape has the in-launch reduction (the last workgroup of a tile row sums that
         // row's slabs, the 2:4 part's included), which saves the separate reduction kernel.
         if ((rc = a24_launch_spmm(stream, Packed_A1, B, ws_a1, M, N, K, Split_K_A1, d.row_blocks, d.waves, d.share_b, K, M,
-                                  mn)) != 0)
+                                  mn, 0, nullptr, nullptr, 0, -1, nullptr, 0, row_major ? 1 : 0)) != 0)
             return rc;
         CallOptions o;
+        o.row_major = row_major;
         o.extra_slabs = Split_K_A1;
         if ((rc = launch_main(stream, Compressed_A2, TileOffsets_A2, B, ws, M, N, K, Split_K_A2, o, K, M, false, C, M,
                               &fused)) != 0)
@@ -676,6 +702,7 @@ extern "C" int HeteroSparse_SpMM_API(void* stream, const void* Packed_A1, const 
         return 0;
     return tcsl_launch_reduce(stream, C, ws, mn, 1, mn, Split_K_A1 + Split_K_A2, 0);
 }
+}  // namespace
 
 extern "C" int HeteroSparse_PackA2(const uint16_t* A2_h, int M, int K, uint32_t** Words, int** Offsets, int* LongestList)
 {
@@ -709,7 +736,7 @@ namespace {
 // not ask for the second kernel), else the reduction kernel follows.
 int a24_split_call(void* stream, const void* Packed_A1, const void* B, long ldb, void* C, long ldc, int M, int N, int K,
                    void* Reduction_Workspace, int Split_K, int row_blocks, int waves, int loads, const void* words,
-                   const void* offsets, int relu, bool separate_reduction)
+                   const void* offsets, int relu, bool separate_reduction, bool row_major)
 {
     const long mn = static_cast<long>(M) * N;
     int page = -1;
@@ -721,18 +748,21 @@ int a24_split_call(void* stream, const void* Packed_A1, const void* B, long ldb,
         page = counter_page(stream);
     }
     int rc = a24_launch_spmm(stream, Packed_A1, B, Reduction_Workspace, M, N, K, Split_K, row_blocks, waves, 1, ldb, M, mn, loads,
-                             words, offsets, page >= 0 ? relu : 0, page, page >= 0 ? C : nullptr, ldc);
+                             words, offsets, page >= 0 ? relu : 0, page, page >= 0 ? C : nullptr, ldc, row_major ? 1 : 0);
     if (rc == 0 && tcsl::CounterPages::recycled(page))
         rc = tcsl_page_mark(page, stream);
     if (page_lock.owns_lock())
         page_lock.unlock();
     if (rc != 0 || page >= 0)
         return rc;
+    if (row_major)  // C is as dense as the slabs: one flat vector
+        return tcsl_launch_reduce(stream, C, static_cast<uint16_t*>(Reduction_Workspace), mn, 1, mn, Split_K, relu);
     return tcsl_launch_reduce(stream, C, static_cast<uint16_t*>(Reduction_Workspace), M, N, ldc, Split_K, relu);
 }
 
 int fused_call(const char* who, void* stream, const void* Packed_A1, const void* A2_Words, const int* A2_Offsets, int LongestList,
-               const void* B, long ldb, void* C, long ldc, int M, int N, int K, void* Reduction_Workspace, int Split_K, int Flags)
+               const void* B, long ldb, void* C, long ldc, int M, int N, int K, void* Reduction_Workspace, int Split_K, int Flags,
+               bool row_major = false)
 {
     if (N != 8 && N != 16 && N != 32 && N != 64) {
         std::printf("MM_Sparse_API Error: Unsupported N dimension %d!\n", N);  // csrc/SpMM_API.cu:192-193
@@ -740,7 +770,8 @@ int fused_call(const char* who, void* stream, const void* Packed_A1, const void*
     }
     // two row blocks per wave, activation tile shared through LDS: the one layout that takes the residual along
     const int loads = (LongestList + 63) / 64;
-    const int waves = (N == 64 && loads >= 5) ? 4 : a24_waves_for(M > 0 ? M : 128, Split_K);  // the former: what fits the registers
+    // (four waves for the longest lists at 64 tokens: what fits the registers)
+    const int waves = (N == 64 && loads >= (row_major ? 4 : 5)) ? 4 : a24_waves_for(M > 0 ? M : 128, Split_K);
     if (!Packed_A1 || !A2_Words || !A2_Offsets || !B || !C || LongestList < 0 || LongestList > HETERO_FUSED_MAX_LIST
         || !a24_shape_ok(M, N, K, Split_K, 2, waves, 1) || (Split_K > 1 && !Reduction_Workspace) || ldb < K || ldc < M
         || ldb % 8 != 0 || ldc % 8 != 0 || (Flags & ~(SPMM_FLAG_RELU | SPMM_FLAG_SEPARATE_REDUCTION))) {
@@ -751,9 +782,10 @@ int fused_call(const char* who, void* stream, const void* Packed_A1, const void*
     const int relu = (Flags & SPMM_FLAG_RELU) ? 1 : 0;
     const long mn = static_cast<long>(M) * N;
     if (Split_K == 1)
-        return a24_launch_spmm(stream, Packed_A1, B, C, M, N, K, 1, 2, waves, 1, ldb, ldc, mn, loads, A2_Words, A2_Offsets, relu);
+        return a24_launch_spmm(stream, Packed_A1, B, C, M, N, K, 1, 2, waves, 1, ldb, ldc, mn, loads, A2_Words, A2_Offsets, relu, -1,
+                               nullptr, 0, row_major ? 1 : 0);
     return a24_split_call(stream, Packed_A1, B, ldb, C, ldc, M, N, K, Reduction_Workspace, Split_K, 2, waves, loads, A2_Words,
-                          A2_Offsets, relu, (Flags & SPMM_FLAG_SEPARATE_REDUCTION) != 0);
+                          A2_Offsets, relu, (Flags & SPMM_FLAG_SEPARATE_REDUCTION) != 0, row_major);
 }
 
 }  // namespace
@@ -773,4 +805,12 @@ extern "C" int HeteroSparse_Fused_SpMM_API_Strided(void* stream, const void* Pac
 {
     return fused_call("HeteroSparse_Fused_SpMM_API_Strided", stream, Packed_A1, A2_Words, A2_Offsets, LongestList, B, ldb, C, ldc,
                       M, N, K, Reduction_Workspace, Split_K, Flags);
+}
+
+extern "C" int HeteroSparse_Fused_SpMM_API_RowMajor(void* stream, const void* Packed_A1, const void* A2_Words,
+                                                    const int* A2_Offsets, int LongestList, const void* B, void* C, int M,
+                                                    int N, int K, void* Reduction_Workspace, int Split_K, int Flags)
+{
+    return fused_call("HeteroSparse_Fused_SpMM_API_RowMajor", stream, Packed_A1, A2_Words, A2_Offsets, LongestList, B, K, C, M, M, N,
+                      K, Reduction_Workspace, Split_K, Flags, true);
 }

@@ -126,7 +126,7 @@ def build_split_layer_on_device(G, torch, dev, h, N, sparsity, seed, weight_std=
 
 class Stack:
     """row_major: every buffer holds [features][N] (this fork's operand layout) instead of one vector per
-    token; the output projection then reads the first h rows of the fused QKV result.  Tiled-CSL weights only."""
+    token; the output projection then reads the first h rows of the fused QKV result."""
 
     def __init__(self, G, torch, layers, h, N, row_major=False):
         self.G, self.torch, self.layers, self.h, self.N, self.row_major = G, torch, layers, h, N, row_major
@@ -145,9 +145,12 @@ class Stack:
     def _product(self, stream, mat, src, ldb, dst, ldc, flags=0):
         it, of, M, K, s = mat
         if self.row_major:
-            if Layer.is_split(mat) or it is None:
-                raise ValueError("the row-major chain takes Tiled-CSL weights only")
-            self.G.SpMM_SplitK_API_RowMajor_Flags(stream, it, of, src, dst, M, self.N, K, self.ws, s, flags)
+            if it is None:
+                raise ValueError("the row-major chain takes encoded weights only")
+            if Layer.is_split(mat):
+                self.G.HeteroSparse_Fused_SpMM_API_RowMajor(stream, it[0], it[1], of[0], of[1], src, dst, M, self.N, K, self.ws, s, flags)
+            else:
+                self.G.SpMM_SplitK_API_RowMajor_Flags(stream, it, of, src, dst, M, self.N, K, self.ws, s, flags)
         elif Layer.is_split(mat):
             self.G.HeteroSparse_Fused_SpMM_API_Strided(stream, it[0], it[1], of[0], of[1], src, ldb, dst, ldc, M, self.N, K,
                                                        self.ws, s, flags)

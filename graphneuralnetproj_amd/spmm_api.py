@@ -67,6 +67,8 @@ EXPORTED_SYMBOLS = (
     "HeteroSparse_DevicePackA2_Words",
     "HeteroSparse_Fused_SpMM_API",
     "HeteroSparse_Fused_SpMM_API_Strided",
+    "HeteroSparse_SpMM_API_RowMajor",
+    "HeteroSparse_Fused_SpMM_API_RowMajor",
 )
 
 
@@ -200,6 +202,11 @@ def load_library():
     lib.HeteroSparse_Fused_SpMM_API_Strided.restype = ctypes.c_int
     lib.HeteroSparse_Fused_SpMM_API_Strided.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int, ctypes.c_void_p, ctypes.c_long,
                                                         ctypes.c_void_p, ctypes.c_long] + [ctypes.c_int] * 3 + [
+        ctypes.c_void_p, ctypes.c_int, ctypes.c_int]
+    lib.HeteroSparse_SpMM_API_RowMajor.restype = ctypes.c_int
+    lib.HeteroSparse_SpMM_API_RowMajor.argtypes = lib.HeteroSparse_SpMM_API.argtypes
+    lib.HeteroSparse_Fused_SpMM_API_RowMajor.restype = ctypes.c_int
+    lib.HeteroSparse_Fused_SpMM_API_RowMajor.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] + [ctypes.c_void_p] * 2 + [ctypes.c_int] * 3 + [
         ctypes.c_void_p, ctypes.c_int, ctypes.c_int]
     lib.HeteroSparse_A1_Partials.restype = ctypes.c_int
     lib.HeteroSparse_A1_Partials.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 7
@@ -541,6 +548,34 @@ def HeteroSparse_Fused_SpMM_API_Strided(stream, Packed_A1, A2_Words, A2_Offsets,
                                                  K_Global, _ptr(Reduction_Workspace), Split_K, Flags)
     if rc != 0:
         raise SpMMError("HeteroSparse_Fused_SpMM_API_Strided", rc, lib.SpMM_GetErrorString(rc).decode())
+    return rc
+
+
+def HeteroSparse_SpMM_API_RowMajor(stream, Packed_A1, Compressed_A2, TileOffsets_A2, B, C, M_Global, N_Global, K_Global,
+                                   Reduction_Workspace, Split_K_A1, Split_K_A2, Flags=0):
+    """HeteroSparse_SpMM_API for row-major operands: B[K][N], C[M][N] (and M x N slabs in the workspace)."""
+    lib = load_library()
+    if stream is not None and not isinstance(stream, int):
+        stream = stream.cuda_stream
+    rc = lib.HeteroSparse_SpMM_API_RowMajor(ctypes.c_void_p(stream) if stream else None, _ptr(Packed_A1), _ptr(Compressed_A2),
+                                            _ptr(TileOffsets_A2), _ptr(B), _ptr(C), M_Global, N_Global, K_Global,
+                                            _ptr(Reduction_Workspace), Split_K_A1, Split_K_A2, Flags)
+    if rc != 0:
+        raise SpMMError("HeteroSparse_SpMM_API_RowMajor", rc, lib.SpMM_GetErrorString(rc).decode())
+    return rc
+
+
+def HeteroSparse_Fused_SpMM_API_RowMajor(stream, Packed_A1, A2_Words, A2_Offsets, LongestList, B, C, M_Global, N_Global, K_Global,
+                                         Reduction_Workspace, Split_K, Flags=0):
+    """HeteroSparse_Fused_SpMM_API for row-major operands (B[K][N], C[M][N]) with Flags (SPMM_FLAG_RELU, ...)."""
+    lib = load_library()
+    if stream is not None and not isinstance(stream, int):
+        stream = stream.cuda_stream
+    rc = lib.HeteroSparse_Fused_SpMM_API_RowMajor(ctypes.c_void_p(stream) if stream else None, _ptr(Packed_A1), _ptr(A2_Words),
+                                                  _ptr(A2_Offsets), LongestList, _ptr(B), _ptr(C), M_Global, N_Global, K_Global,
+                                                  _ptr(Reduction_Workspace), Split_K, Flags)
+    if rc != 0:
+        raise SpMMError("HeteroSparse_Fused_SpMM_API_RowMajor", rc, lib.SpMM_GetErrorString(rc).decode())
     return rc
 
 

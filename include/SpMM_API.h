@@ -447,6 +447,29 @@ SPMM_EXPORT int HeteroSparse_Fused_SpMM_API_Strided(void* stream, const void* Pa
                                                     long ldc, int M_Global, int N_Global, int K_Global,
                                                     void* Reduction_Workspace, int Split_K, int Flags);
 
+/*
+ * The two calls above for row-major operands, the layout of this checkout's own hybrid kernel and
+ * benchmark (csrc/SpMM_Kernel.cuh:372-374 for B, :731-734 for the output;
+ * kernel_benchmark/spmm_test.cu:137-141,474,569-576): B[k*N + n] (K x N), C[m*N + n] (M x N), both
+ * dense, and every slab of partial sums in the workspace M x N as well.  The weight operands are the
+ * same records, Tiled-CSL residual or residual lists as for the column-major calls.
+ *   HeteroSparse_SpMM_API_RowMajor        arguments, checks and return codes of HeteroSparse_SpMM_API;
+ *   HeteroSparse_Fused_SpMM_API_RowMajor  those of HeteroSparse_Fused_SpMM_API plus Flags (0 or a sum of
+ *                                         SPMM_FLAG_RELU and SPMM_FLAG_SEPARATE_REDUCTION).  A chain of
+ *                                         layers needs no strides in this layout: a result is the next
+ *                                         product's B as it stands.
+ * The 2:4 kernel stages each unit's 128 x N activation block in LDS as it sits in memory and reads it
+ * back with the transposing LDS read, as the Tiled-CSL kernel does for SpMM_SplitK_API_RowMajor.
+ */
+SPMM_EXPORT int HeteroSparse_SpMM_API_RowMajor(void* stream, const void* Packed_A1, const void* Compressed_A2,
+                                               const int* TileOffsets_A2, const void* B, void* C, int M_Global,
+                                               int N_Global, int K_Global, void* Reduction_Workspace, int Split_K_A1,
+                                               int Split_K_A2, int Flags);
+SPMM_EXPORT int HeteroSparse_Fused_SpMM_API_RowMajor(void* stream, const void* Packed_A1, const void* A2_Words,
+                                                     const int* A2_Offsets, int LongestList, const void* B, void* C,
+                                                     int M_Global, int N_Global, int K_Global, void* Reduction_Workspace,
+                                                     int Split_K, int Flags);
+
 #ifdef __cplusplus
 }
 #endif

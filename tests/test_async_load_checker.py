@@ -169,4 +169,6 @@ def test_built_sparse_mfma_kernels_pass():
         pytest.skip("library not built in this tree")
     r = subprocess.run([sys.executable, CHECKER, asm, "a24_spmm_shared_b_kernel"], capture_output=True, text=True)
     assert r.returncode == 0, r.stdout
-    assert r.stdout.count("ok ") == 41  # 2 + 5 + 5 launch shapes for 64, 32 and up to 16 tokens, and 9 + 10 + 10 that take the residual along
+    # column-major: 2 + 5 + 5 launch shapes for 64, 32 and up to 16 tokens, and 9 + 10 + 10 that take the residual along;
+    # row-major (two row blocks per wave only): 2 + 2 + 2 and 8 + 10 + 10
+    assert r.stdout.count("ok ") == 41 + 34

@@ -251,6 +251,12 @@ def test_exact_two_to_four_part_and_residual(spmm, oracle, M, K, sparsity):
         spmm.HeteroSparse_SpMM_API(stream, d_packed, d_items2, d_offs2, d_B[:N], d_C, M, N, K, d_W, s1[N], s2[N])
         torch.cuda.synchronize()
         _assert_identical(d_C.cpu().numpy(), total.astype(np.float16), f"two kernels {M}x{K} N={N}")
+        d_Bt = d_B[:N].t().contiguous()   # the same call on row-major operands: B[K][N], C[M][N], M x N slabs
+        d_Ct = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda:0")
+        d_W.fill_(float("nan"))
+        spmm.HeteroSparse_SpMM_API_RowMajor(stream, d_packed, d_items2, d_offs2, d_Bt, d_Ct, M, N, K, d_W, s1[N], s2[N])
+        torch.cuda.synchronize()
+        _assert_identical(d_Ct.t().contiguous().cpu().numpy(), total.astype(np.float16), f"two kernels, row-major {M}x{K} N={N}")
         if longest > spmm.HETERO_FUSED_MAX_LIST:
             continue
         # one launch: per batch of units one fp16 slab of both parts' sum (no rounding with one batch)
@@ -263,3 +269,7 @@ def test_exact_two_to_four_part_and_residual(spmm, oracle, M, K, sparsity):
         spmm.HeteroSparse_Fused_SpMM_API(stream, d_packed, d_words, d_lists, longest, d_B[:N], d_C, M, N, K, d_W, s1[N])
         torch.cuda.synchronize()
         _assert_identical(d_C.cpu().numpy(), total.astype(np.float16), f"one launch {M}x{K} N={N}")
+        d_Ct.fill_(float("nan"))
+        spmm.HeteroSparse_Fused_SpMM_API_RowMajor(stream, d_packed, d_words, d_lists, longest, d_Bt, d_Ct, M, N, K, d_W, s1[N])
+        torch.cuda.synchronize()
+        _assert_identical(d_Ct.t().contiguous().cpu().numpy(), total.astype(np.float16), f"one launch, row-major {M}x{K} N={N}")

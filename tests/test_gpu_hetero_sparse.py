@@ -568,9 +568,11 @@ def test_fused_strided_operands_and_clamp(spmm, oracle, split_k):
             spmm.HeteroSparse_Fused_SpMM_API_Strided(None, d, d, d, 10, d, ldb_bad, d, ldc_bad, M, N, K, d, 1, 0)
 
 
-def test_split_decoder_stack_matches_cpu_chain(spmm, oracle):
+@pytest.mark.parametrize("row_major", [False, True])
+def test_split_decoder_stack_matches_cpu_chain(spmm, oracle, row_major):
     """Three chained blocks with every weight split into 2:4 records + residual lists on the GPU,
-    each product one launch, against the same chain on the CPU; and replays of the captured chain."""
+    each product one launch, against the same chain on the CPU; and replays of the captured chain.
+    row_major: every buffer [features][tokens], products through HeteroSparse_Fused_SpMM_API_RowMajor."""
     torch = _torch()
     from graphneuralnetproj_amd import decoder_stack as DS
 
@@ -586,11 +588,13 @@ def test_split_decoder_stack_matches_cpu_chain(spmm, oracle):
             assert rows.size == M  # every row: the whole matrix comes back, in row order
             d[name] = vals
         dense.append(d)
-    stack = DS.Stack(spmm, torch, layers, h, N)
+    stack = DS.Stack(spmm, torch, layers, h, N, row_major=row_major)
     x0 = spmm.synth_activations(N, h, seed=98)
     x0_d = torch.from_numpy(x0.view(np.int16)).to(dev).view(torch.float16)
+    if row_major:
+        x0_d = x0_d.t().contiguous()
     stack.x[0].copy_(x0_d)
-    print(f"[gpu case] split decoder stack h={h} N={N} layers={nlayers}", flush=True)
+    print(f"[gpu case] split decoder stack h={h} N={N} layers={nlayers} row_major={row_major}", flush=True)
     out = stack.step(torch.cuda.current_stream())
     torch.cuda.synchronize()
     got = out.clone()
@@ -603,7 +607,8 @@ def test_split_decoder_stack_matches_cpu_chain(spmm, oracle):
         x = f16(oracle.gemm_f32(d["ffn2"], f))
     xr = x.astype(np.float32)
     assert np.abs(xr).max() > 1e-3, "the reference chain must not have collapsed to zero"
-    err = np.abs(got.cpu().numpy().astype(np.float32) - xr)
+    got_h = (got.t() if row_major else got).cpu().numpy().astype(np.float32)
+    err = np.abs(got_h - xr)
     scale = np.maximum(np.abs(xr), np.sqrt(np.mean(xr * xr)))
     assert (err <= 3 * (ATOL + RTOL * scale)).all(), err.max()  # twelve products, fp16 between them
     g = torch.cuda.CUDAGraph()
@@ -681,3 +686,127 @@ def test_fused_call_sums_its_slabs_in_the_launch_bit_for_bit(spmm, oracle, M, K,
         C1 = run_hybrid(spmm, spmm.HeteroSparse_PackA1(A1), None, None, Bh, M, N, K, split_k, 0)
         assert_close(C1, oracle.gemm_f32(A1, Bh))
 
+
+
+# ---------------------------------------------------------------------------------------------
+# row-major operands (B[K][N], C[M][N]): this fork's own layout, csrc/SpMM_Kernel.cuh:372-374,731-734
+
+
+def run_fused_row_major(spmm, packed, words, offs, longest, B, M, N, K, split_k, flags=0):
+    """B is the usual [N][K] host array; the call gets its transpose and the result comes back as [N][M]."""
+    torch = _torch()
+    d_p, d_w, d_o = _dev(packed), _dev(words), _dev(offs)
+    d_Bt = _dev(B).view(torch.float16).t().contiguous()
+    d_Ct = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda:0")
+    d_W = torch.full((max(split_k, 1), M, N), float("nan"), dtype=torch.float16, device="cuda:0")
+    print(f"[gpu case] fused row-major M={M} N={N} K={K} split_k={split_k} longest={longest} flags={flags}", flush=True)
+    spmm.HeteroSparse_Fused_SpMM_API_RowMajor(torch.cuda.current_stream(), d_p, d_w, d_o, longest, d_Bt, d_Ct, M, N, K, d_W,
+                                              split_k, flags)
+    torch.cuda.synchronize()
+    return d_Ct.t().contiguous().cpu().numpy()
+
+
+def run_hybrid_row_major(spmm, packed, items, offsets, B, M, N, K, s1, s2, flags=0):
+    torch = _torch()
+    d_p = _dev(packed)
+    d_items = _dev(items) if items is not None else None
+    d_offs = _dev(offsets) if offsets is not None else None
+    d_Bt = _dev(B).view(torch.float16).t().contiguous()
+    d_Ct = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda:0")
+    d_W = torch.full((s1 + s2, M, N), float("nan"), dtype=torch.float16, device="cuda:0")
+    print(f"[gpu case] hybrid row-major M={M} N={N} K={K} split_k={s1}/{s2} flags={flags}", flush=True)
+    spmm.HeteroSparse_SpMM_API_RowMajor(torch.cuda.current_stream(), d_p, d_items, d_offs, d_Bt, d_Ct, M, N, K, d_W, s1, s2, flags)
+    torch.cuda.synchronize()
+    return d_Ct.t().contiguous().cpu().numpy()
+
+
+@pytest.mark.parametrize("N", [8, 16, 32, 64])
+def test_row_major_layout_one_hot(spmm, oracle, N):
+    """Rows, columns and tokens of the row-major entries, through both parts: distinct exactly
+    representable integers and one-hot activations, so C[m][n] must equal A[m][k_n] exactly (the
+    staging of the K x N block, the transposing reads and the M x N stores all have to be right)."""
+    M, K = 256, 384
+    rng = np.random.default_rng(40 + N)
+    A = np.zeros((M, K), dtype=np.float16)
+    mask = rng.random((M, K)) < 0.45
+    vals = (np.arange(M * K).reshape(M, K) % 1999 + 1).astype(np.float16)
+    A[mask] = vals[mask]
+    A1, A2 = oracle.decompose(A)
+    packed = spmm.HeteroSparse_PackA1(A1)
+    words, offs, longest = spmm.HeteroSparse_PackA2(A2)
+    items, offsets = spmm.InitSparseMatrixA_API(A2)
+    for trial in range(3):
+        ks = rng.permutation(K)[:N]
+        B = np.zeros((N, K), dtype=np.float16)
+        B[np.arange(N), ks] = 1.0
+        want = A[:, ks].T.view(np.uint16)
+        for split_k in (1, 3):
+            C = run_fused_row_major(spmm, packed, words, offs, longest, B, M, N, K, split_k)
+            assert np.array_equal(C.view(np.uint16), want), (trial, split_k)
+        C = run_hybrid_row_major(spmm, packed, items, offsets, B, M, N, K, 1, 2)
+        assert np.array_equal(C.view(np.uint16), want), trial
+        C = run_hybrid_row_major(spmm, packed, None, None, B, M, N, K, 3, 0)   # the 2:4 part alone, three batches
+        assert np.array_equal(C.view(np.uint16), A1[:, ks].T.view(np.uint16)), trial
+        C = run_hybrid_row_major(spmm, packed, None, None, B, M, N, K, 1, 0)   # ... and one
+        assert np.array_equal(C.view(np.uint16), A1[:, ks].T.view(np.uint16)), trial
+
+
+@pytest.mark.parametrize("sparsity", [0.45, 0.6, 0.8, 0.95])
+@pytest.mark.parametrize("N", [8, 16, 32, 64])
+@pytest.mark.parametrize("M,K,split_k", [(384, 1152, 1), (512, 1024, 2), (2048, 640, 5)])
+def test_row_major_fused_equals_column_major_bit_for_bit(spmm, oracle, sparsity, N, M, K, split_k):
+    """The one-launch call in both layouts: every element takes the same products in the same order
+    (units, steps and the order of the two parts do not depend on the layout), so the results are
+    the same bits, with and without the clamp and the in-launch sum; and they match the oracle."""
+    A = spmm.synth_weights(M, K, sparsity, False, seed=M + K + N)
+    A1, A2 = spmm.HeteroSparse_Decompose(A)
+    packed = spmm.HeteroSparse_PackA1(A1)
+    words, offs, longest = spmm.HeteroSparse_PackA2(A2)
+    B = spmm.synth_activations(N, K, seed=71)
+    col = run_fused(spmm, packed, words, offs, longest, B, M, N, K, split_k)
+    assert_close(col, oracle.gemm_f32(A, B))
+    for flags in (0, spmm.SPMM_FLAG_SEPARATE_REDUCTION):
+        row = run_fused_row_major(spmm, packed, words, offs, longest, B, M, N, K, split_k, flags)
+        assert np.array_equal(row.view(np.uint16), col.view(np.uint16)), flags
+    row = run_fused_row_major(spmm, packed, words, offs, longest, B, M, N, K, split_k, spmm.SPMM_FLAG_RELU)
+    assert np.array_equal(row, np.maximum(col, np.float16(0)))
+
+
+@pytest.mark.parametrize("sparsity", [0.5, 0.7])
+@pytest.mark.parametrize("N", [8, 16, 64])
+def test_row_major_hybrid_vs_oracle(spmm, oracle, sparsity, N):
+    """The two-kernel call in the row-major layout (the residual on the Tiled-CSL kernel's row-major
+    form, which adds all slabs up, the 2:4 part's included), one and two streams."""
+    M, K = 1024, 2048
+    A = spmm.synth_weights(M, K, sparsity, False, seed=81 + N)
+    A1, A2 = spmm.HeteroSparse_Decompose(A)
+    packed = spmm.HeteroSparse_PackA1(A1)
+    items, offsets = spmm.InitSparseMatrixA_API(A2)
+    B = spmm.synth_activations(N, K, seed=82)
+    ref = oracle.gemm_f32(A, B)
+    for s1, s2, flags in ((1, 1, 0), (2, 4, 0), (4, 3, 0), (2, 2, spmm.HETERO_FLAG_TWO_STREAMS)):
+        assert_close(run_hybrid_row_major(spmm, packed, items, offsets, B, M, N, K, s1, s2, flags), ref)
+
+
+def test_row_major_full_size_and_rejects(spmm, oracle):
+    """OPT-30B FFN1 at 60 %, N = 16 and 64, the one-launch call in the row-major layout at full size:
+    the same bits as the column-major call.  And what the entry refuses."""
+    torch = _torch()
+    M, K = 28672, 7168
+    A = spmm.synth_weights(M, K, 0.6, False, seed=23)
+    A1, A2 = spmm.HeteroSparse_Decompose(A)
+    packed = spmm.HeteroSparse_PackA1(A1)
+    words, offs, longest = spmm.HeteroSparse_PackA2(A2)
+    for N in (16, 64):
+        B = spmm.synth_activations(N, K, seed=3)
+        s = spmm.HeteroSparse_SuggestSplitK(M, N, K)
+        col = run_fused(spmm, packed, words, offs, longest, B, M, N, K, s)
+        row = run_fused_row_major(spmm, packed, words, offs, longest, B, M, N, K, s)
+        assert np.array_equal(row.view(np.uint16), col.view(np.uint16))
+    d = torch.zeros(64, dtype=torch.int32, device="cuda:0")
+    for bad in (dict(M=200), dict(K=576), dict(N=24), dict(flags=8)):
+        a = dict(M=256, K=512, N=16, flags=0)
+        a.update(bad)
+        with pytest.raises(spmm.SpMMError):
+            spmm.HeteroSparse_Fused_SpMM_API_RowMajor(torch.cuda.current_stream(), d, d, d, 10, d, d, a["M"], a["N"], a["K"], d, 1,
+                                                      a["flags"])
