@@ -284,6 +284,8 @@ def sweep(G, lib, torch, dev, sptr, with_stack):
     torch.cuda.empty_cache()
     for sparsity in (0.6, 0.7):
         out.append(split_case(G, lib, torch, dev, sptr, "opt30b_ffn1", 16, sparsity))
+    # row-skewed: residual lists of up to several hundred words, beyond what travels with the records
+    out.append(split_case(G, lib, torch, dev, sptr, "opt30b_ffn1", 16, 0.6, skew=True))
     if with_stack:
         out.append(stack_step(G, torch, dev))
         # the same stack at a sparsity where the fork's split pays, in both forms
@@ -292,12 +294,12 @@ def sweep(G, lib, torch, dev, sptr, with_stack):
     return out
 
 
-def split_case(G, lib, torch, dev, sptr, workload, N, sparsity):
+def split_case(G, lib, torch, dev, sptr, workload, N, sparsity, skew=False):
     """The fork's split of a weight into a 2:4 part and a residual, at a sparsity where it can pay:
     plain Tiled-CSL, the two-kernel call and the one-launch call on the same weight, whole calls
     between two events, weights rotated over three copies."""
     M, K = WORKLOADS[workload][:2]
-    A = G.synth_weights(M, K, sparsity, False, seed=1234)
+    A = G.synth_weights(M, K, sparsity, skew, seed=1234)
     A1, A2 = G.HeteroSparse_Decompose(A)
     items, offsets = G.InitSparseMatrixA_API(A)
     del A
@@ -339,21 +341,28 @@ def split_case(G, lib, torch, dev, sptr, workload, N, sparsity):
         check(lib.HeteroSparse_Fused_SpMM_API(sptr, p["packed"][i % copies], p["words"][i % copies], p["lists"][i % copies], longest,
                                               p_B, p_C, M, N, K, p_W, s_a1), "HeteroSparse_Fused_SpMM_API")
 
+    def one_row_major(i):  # the same buffers hold either layout's elements
+        check(lib.HeteroSparse_Fused_SpMM_API_RowMajor(sptr, p["packed"][i % copies], p["words"][i % copies], p["lists"][i % copies],
+                                                       longest, p_B, p_C, M, N, K, p_W, s_a1, 0), "HeteroSparse_Fused_SpMM_API_RowMajor")
+
     res = {}
     outputs = {}
-    for name, fn in (("tiled_csl", csl), ("two_kernels", two), ("one_launch", one)):
-        if name == "one_launch" and longest > G.HETERO_FUSED_MAX_LIST:
+    for name, fn in (("tiled_csl", csl), ("two_kernels", two), ("one_launch", one), ("one_launch_row_major", one_row_major)):
+        if name.startswith("one_launch") and longest > G.HETERO_FUSED_MAX_LIST:
             res[name] = None
             continue
         prewarm(fn, torch, 0.1)
         res[name] = float(np.median([events_ms(lib, sptr, fn, 100) for _ in range(3)])) / 100
         torch.cuda.synchronize()
-        outputs[name] = d_C.float().cpu().numpy()
+        if name != "one_launch_row_major":  # (its operands are the other layout's bytes: timing only)
+            outputs[name] = d_C.float().cpu().numpy()
     ref = outputs["tiled_csl"]
     agree = all(bool((np.abs(o - ref) <= 2e-2 + 2e-2 * np.abs(ref)).all()) for o in outputs.values())
     one_bytes = packed.nbytes + 4 * int(list_offsets[-1])
     best = res["one_launch"] or res["two_kernels"]
-    return {"case": f"ffn1_{int(sparsity * 100)}pct_2to4_plus_residual", "M": M, "K": K, "N": N, "sparsity": sparsity,
+    return {"case": f"ffn1_{int(sparsity * 100)}pct{'_skewed' if skew else ''}_2to4_plus_residual", "M": M, "K": K, "N": N,
+            "sparsity": sparsity, "row_skewed": skew, "longest_residual_list": longest,
+            "one_launch_row_major_ms": res["one_launch_row_major"],
             "tiled_csl_bytes": 16 * int(offsets[-1]), "records_bytes": packed.nbytes, "residual_list_bytes": 4 * int(list_offsets[-1]),
             "tiled_csl_ms": res["tiled_csl"], "two_kernels_ms": res["two_kernels"], "one_launch_ms": res["one_launch"],
             "split_k": {"tiled_csl": s_csl, "records": s_a1, "residual": s_res}, "outputs_agree": agree,
@@ -409,22 +418,22 @@ def stack_step(G, torch, dev, layers=64, h=9216, N=16, sparsity=0.8, split=False
     weight_bytes = sum(L.bytes() for L in blocks)
     ms = min(eager_ms, graph_ms) if graph_ms else eager_ms
     row_major_ms = None
-    if not split:  # the same weights with the activations in this fork's layout, [features][tokens]
-        del stack, g
-        stack = DS.Stack(G, torch, blocks, h, N, row_major=True)
-        stack.x[0].copy_(x0.t())
+    # the same weights with the activations in this fork's layout, [features][tokens]
+    del stack, g
+    stack = DS.Stack(G, torch, blocks, h, N, row_major=True)
+    stack.x[0].copy_(x0.t())
+    for _ in range(5):
+        stack.step(stream)
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(5):
+        t0 = time.perf_counter()
         for _ in range(5):
             stack.step(stream)
         torch.cuda.synchronize()
-        times = []
-        for _ in range(5):
-            t0 = time.perf_counter()
-            for _ in range(5):
-                stack.step(stream)
-            torch.cuda.synchronize()
-            times.append((time.perf_counter() - t0) * 1e3 / 5)
-        row_major_ms = float(np.median(times))
-        g = None
+        times.append((time.perf_counter() - t0) * 1e3 / 5)
+    row_major_ms = float(np.median(times))
+    g = None
     del stack, blocks, g
     torch.cuda.empty_cache()
     case = "decoder_stack" if sparsity == 0.8 and not split else f"decoder_stack_{int(sparsity * 100)}pct" + ("_split" if split else "")

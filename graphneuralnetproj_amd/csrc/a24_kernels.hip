@@ -241,7 +241,8 @@ constexpr int kRowBytes = 272;
 // With RL > 0 the same launch also multiplies the residual (what the split leaves beyond two kept
 // values per group of four), so that C = A1*B + A2*B costs one pass over the activations instead of
 // two kernels and a sum.  The residual comes as one list of words per record (a24_format.h:
-// fp16 value | byte address in a 16 x 128 image << 16), at most RL * 64 words each.  A wave
+// fp16 value | byte address in a 16 x 128 image << 16); RL rounds of 64 words travel with the unit's
+// records, and what a longer list holds beyond them is fetched inside the unit's multiplication.  A wave
 // scatters a list into its own 4 KiB LDS image (ds_write_b16; lanes past the end repeat the last
 // word), reads the image back as dense MFMA operands, writes zeros where it wrote values, and runs
 // v_mfma_f32_16x16x32_f16 on the same activation fragments and accumulators as the sparse
@@ -360,6 +361,7 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
         unsigned w[RB][RLA];  // residual words of the unit's RB lists
         int next;             // lane j <= RB: offsets[first record of the unit after this one + j]
         int count[RB];        // words in each list (the same in every lane)
+        int start[RB];        // where each list starts in `words`
     };
     constexpr int kLoadsA = (3 + RL) * RB;      // loads of one unit's records and lists per lane
     constexpr int kLoadsHead = RL > 0 ? 1 : 0;  // the offsets load that leads a unit's loads
@@ -386,6 +388,7 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
             for (int r = 0; r < RB; r++) {
                 const int n = o[r + 1] - o[r];
                 x.count[r] = n;
+                x.start[r] = o[r];
                 const int last = n > 0 ? n - 1 : 0;
 #pragma unroll
                 for (int i = 0; i < RL; i++) {
@@ -445,13 +448,32 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
                     for (int i = 0; i < RL; i++)
                         if (i == 0 || n > i * kWave)
                             *reinterpret_cast<unsigned short*>(image + (x.w[r][i] >> 16)) = static_cast<unsigned short>(x.w[r][i]);
+                    // A list longer than the RL rounds that travel with the unit (a block of a
+                    // row-skewed weight; a residual block holds up to 1024 words): the rest is fetched
+                    // here, with ordinary loads, which wait for everything this wave has in flight.
+                    // That stalls the wave's pipeline once per such list; the constant waits further
+                    // on stay right, since they only ever ask for fewer loads to be outstanding.
+                    const bool longer = n > RL * kWave;
+                    if (longer) {
+                        for (int at0 = RL * kWave; at0 < n; at0 += kWave) {
+                            const int at = at0 + lane;
+                            const unsigned w = words[x.start[r] + (at < n ? at : n - 1)];
+                            *reinterpret_cast<unsigned short*>(image + (w >> 16)) = static_cast<unsigned short>(w);
+                        }
+                    }
 #pragma unroll
                     for (int s = 0; s < 4; s++)
                         dense[r][s] = *reinterpret_cast<const half8*>(image + img_row + (((s * 4 + (lane >> 4)) ^ (lane & 15)) << 4));
+                    if (longer) {  // the extra words are gone: clear the whole image (as much LDS traffic as four rounds)
 #pragma unroll
-                    for (int i = 0; i < RL; i++)
-                        if (i == 0 || n > i * kWave)
-                            *reinterpret_cast<unsigned short*>(image + (x.w[r][i] >> 16)) = 0;
+                        for (int i = 0; i < kImageBytes / (kWave * 16); i++)
+                            *reinterpret_cast<u32x4*>(image + (i * kWave + lane) * 16) = u32x4{0u, 0u, 0u, 0u};
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < RL; i++)
+                            if (i == 0 || n > i * kWave)
+                                *reinterpret_cast<unsigned short*>(image + (x.w[r][i] >> 16)) = 0;
+                    }
                 }
             }
         }
@@ -718,7 +740,8 @@ int launch_nt(hipStream_t s, const void* packed, const void* B, void* out, int M
 // Batch b of ceil((K/128)/split_k) units writes fp16 [N][ldo] to out + b * slab.  The caller has
 // checked: M % (16 * rb) == 0 (share_b: M % (16 * rb * waves) == 0), K % 128 == 0, N in {8, 16, 32, 64}, no batch empty, pointers set.
 // residual_loads > 0 (share_b with rb == 2 only): the launch also multiplies the residual lists
-// words / offsets, none longer than 64 * residual_loads words.  relu (share_b only): negative
+// words / offsets; residual_loads rounds of 64 words travel with the records, a longer list's rest is
+// fetched where it is needed.  relu (share_b only): negative
 // results are written as zero (for a launch that writes the finished result).
 // fuse_page >= 0 (share_b, split_k > 1, ldo == M, slab == M * N): the launch adds its slabs up into
 // fused_out (token stride ldc) itself, counting arrivals on that page of the library's counters.

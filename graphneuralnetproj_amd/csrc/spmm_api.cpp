@@ -769,7 +769,10 @@ int fused_call(const char* who, void* stream, const void* Packed_A1, const void*
         return tcsl_error_unknown();
     }
     // two row blocks per wave, activation tile shared through LDS: the one layout that takes the residual along
-    const int loads = (LongestList + 63) / 64;
+    // up to five rounds of 64 words travel with a unit's records; what a longer list holds beyond them
+    // is fetched where it is needed (a24_kernels.hip)
+    const int rounds = (LongestList + 63) / 64;
+    const int loads = rounds < HETERO_FUSED_PIPELINED_ROUNDS ? rounds : HETERO_FUSED_PIPELINED_ROUNDS;
     // (four waves for the longest lists at 64 tokens: what fits the registers)
     const int waves = (N == 64 && loads >= (row_major ? 4 : 5)) ? 4 : a24_waves_for(M > 0 ? M : 128, Split_K);
     if (!Packed_A1 || !A2_Words || !A2_Offsets || !B || !C || LongestList < 0 || LongestList > HETERO_FUSED_MAX_LIST

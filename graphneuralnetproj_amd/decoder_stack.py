@@ -115,7 +115,7 @@ def build_split_layer_on_device(G, torch, dev, h, N, sparsity, seed, weight_std=
         records, residual = G.split_pack_on_device(A)
         words, offsets, longest = G.pack_residual_on_device(residual)
         if longest > G.HETERO_FUSED_MAX_LIST:
-            raise ValueError(f"{name}: a residual list of {longest} words; the one-launch product takes {G.HETERO_FUSED_MAX_LIST}")
+            raise ValueError(f"{name}: a residual list of {longest} words: more than a residual can hold ({G.HETERO_FUSED_MAX_LIST})")
         mats[name] = ((records, words), (offsets, longest), M, K, G.HeteroSparse_SuggestSplitK(M, N, K))
         if sample_rows:
             rows = torch.randperm(M, generator=gen, device=dev)[:sample_rows].sort().values

@@ -498,7 +498,8 @@ def HeteroSparse_SpMM_API(stream, Packed_A1, Compressed_A2, TileOffsets_A2, B, C
     return rc
 
 
-HETERO_FUSED_MAX_LIST = 320
+HETERO_FUSED_MAX_LIST = 1024  # include/SpMM_API.h: what a block of a residual can hold
+HETERO_FUSED_PIPELINED_ROUNDS = 5
 
 
 def HeteroSparse_PackA2(A2_h, M=None, K=None):

@@ -402,8 +402,11 @@ SPMM_EXPORT int HeteroSparse_A1_Partials(void* stream, const void* Packed_A1, co
  * HeteroSparse_Fused_SpMM_API: C = A1*B + A2*B, one kernel (plus the reduction kernel when
  * Split_K > 1: Reduction_Workspace then holds Split_K*M*N fp16 values; HeteroSparse_SuggestSplitK).
  * Device pointers; B[N][K], C[N][M] as for SpMM_SplitK_API.  LongestList as HeteroSparse_PackA2 gave
- * it, at most HETERO_FUSED_MAX_LIST (uniform sparsity of 50 % and more stays below; a matrix with
- * denser rows has longer lists and goes through HeteroSparse_SpMM_API instead).  Returns a
+ * it, at most HETERO_FUSED_MAX_LIST = 1024, which is what a block of a residual can hold, so every
+ * residual is accepted.  Lists of up to 320 words (uniform sparsity of 50 % and more stays below) travel
+ * with the records' own loads; the words of a longer list (a matrix with some dense rows, e.g.
+ * Beta(2,8)-skewed row densities) beyond the 320th are fetched where they are needed, which stalls that
+ * wave once per such list: correct at any length, fastest when long lists are rare.  Returns a
  * hipError_t value: hipErrorUnknown for N outside {8, 16, 32, 64}; hipErrorInvalidValue for M % 128,
  * K % 128, an empty batch, a list too long, a missing pointer.  Only enqueues work on `stream`.
  */
@@ -428,7 +431,8 @@ SPMM_EXPORT int HeteroSparse_DevicePackA2_Offsets(void* stream, const void* A2_d
 SPMM_EXPORT int HeteroSparse_DevicePackA2_Words(void* stream, const void* A2_d, int M_Global, int K_Global,
                                                 const int* Offsets_d, void* Words_d);
 
-#define HETERO_FUSED_MAX_LIST 320
+#define HETERO_FUSED_MAX_LIST 1024       /* what a 16 x 128 block of a residual can hold: two of every four */
+#define HETERO_FUSED_PIPELINED_ROUNDS 5  /* rounds of 64 words that travel with a unit's records */
 SPMM_EXPORT int HeteroSparse_PackA2(const uint16_t* A2_h, int M_Global, int K_Global, uint32_t** Words, int** Offsets,
                                     int* LongestList);
 SPMM_EXPORT int HeteroSparse_Fused_SpMM_API(void* stream, const void* Packed_A1, const void* A2_Words, const int* A2_Offsets,

@@ -419,18 +419,39 @@ def test_fused_rejects(spmm):
         spmm.HeteroSparse_Fused_SpMM_API(None, d, d, d, 10, d, d, 256, 16, 512, None, 2)
 
 
-def test_fused_row_skewed_weight_has_lists_too_long(spmm):
-    """Beta(2, 8) row densities leave blocks with more than 320 residual values: the packer reports
-    it and the one-launch entry refuses; such a weight goes through HeteroSparse_SpMM_API."""
-    torch = _torch()
+@pytest.mark.parametrize("N", [8, 16, 32, 64])
+@pytest.mark.parametrize("sparsity,skew", [(0.5, True), (0.3, False), (0.1, False)])
+def test_fused_lists_longer_than_the_pipelined_rounds(spmm, oracle, N, sparsity, skew):
+    """Beta(2, 8) row densities (and a nearly dense weight) leave blocks with more than 320 residual
+    values, up to the 1024 a block can hold: the first five rounds of such a list travel with the
+    records, the rest is fetched inside the multiplication.  Both layouts, one and three batches,
+    against the oracle; exact one-hot probe of where every word lands."""
     M, K = 1024, 1024
-    A = spmm.synth_weights(M, K, 0.5, True, seed=3)
-    _, A2 = spmm.HeteroSparse_Decompose(A)
+    A = spmm.synth_weights(M, K, sparsity, skew, seed=3)
+    A1, A2 = spmm.HeteroSparse_Decompose(A)
+    packed = spmm.HeteroSparse_PackA1(A1)
     words, offs, longest = spmm.HeteroSparse_PackA2(A2)
-    assert longest > spmm.HETERO_FUSED_MAX_LIST
-    d = torch.zeros(1 << 12, dtype=torch.int32, device="cuda:0")
-    with pytest.raises(spmm.SpMMError):
-        spmm.HeteroSparse_Fused_SpMM_API(None, d, d, d, longest, d, d, M, 16, K, d, 1)
+    lengths = np.diff(offs)
+    assert longest > 64 * spmm.HETERO_FUSED_PIPELINED_ROUNDS and longest <= spmm.HETERO_FUSED_MAX_LIST
+    assert (lengths <= 64 * spmm.HETERO_FUSED_PIPELINED_ROUNDS).any() or not skew  # short and long lists side by side
+    B = spmm.synth_activations(N, K, seed=5)
+    ref = oracle.gemm_f32(A, B)
+    for split_k in (1, 3):
+        col = run_fused(spmm, packed, words, offs, longest, B, M, N, K, split_k)
+        assert_close(col, ref)
+        row = run_fused_row_major(spmm, packed, words, offs, longest, B, M, N, K, split_k)
+        assert np.array_equal(row.view(np.uint16), col.view(np.uint16))
+    # every element of the weight, whichever part and whichever round of its list holds it
+    ints = np.where(A != 0, (np.arange(M * K).reshape(M, K) % 1999 + 1).astype(np.float16), np.float16(0))
+    I1, I2 = oracle.decompose(ints)
+    p1 = spmm.HeteroSparse_PackA1(I1)
+    w2, o2, l2 = spmm.HeteroSparse_PackA2(I2)
+    rng = np.random.default_rng(N)
+    ks = rng.permutation(K)[:N]
+    onehot = np.zeros((N, K), dtype=np.float16)
+    onehot[np.arange(N), ks] = 1.0
+    C = run_fused(spmm, p1, w2, o2, l2, onehot, M, N, K, 1)
+    assert np.array_equal(C.view(np.uint16), ints[:, ks].T.view(np.uint16))
 
 
 def test_fused_full_size_sampled_rows(spmm, oracle):
@@ -810,3 +831,29 @@ def test_row_major_full_size_and_rejects(spmm, oracle):
         with pytest.raises(spmm.SpMMError):
             spmm.HeteroSparse_Fused_SpMM_API_RowMajor(torch.cuda.current_stream(), d, d, d, 10, d, d, a["M"], a["N"], a["K"], d, 1,
                                                       a["flags"])
+
+
+def test_fused_row_skewed_weight_full_size(spmm, oracle):
+    """OPT-30B FFN1 with Beta(2, 8) row densities at 60 % sparsity, N = 16, through the one-launch call:
+    some blocks' lists exceed what travels with the records.  The rows of the blocks with the longest
+    lists and random rows against the oracle, every row against the two-kernel call."""
+    M, K, N = 28672, 7168, 16
+    A = spmm.synth_weights(M, K, 0.6, True, seed=29)
+    A1, A2 = spmm.HeteroSparse_Decompose(A)
+    packed = spmm.HeteroSparse_PackA1(A1)
+    words, offs, longest = spmm.HeteroSparse_PackA2(A2)
+    assert 64 * spmm.HETERO_FUSED_PIPELINED_ROUNDS < longest <= spmm.HETERO_FUSED_MAX_LIST
+    units = K // 128
+    lengths = np.diff(offs).reshape(M // 128, units, 8)  # lists are numbered by group of eight row blocks, unit, block
+    per_block = lengths.max(axis=1).reshape(-1)           # the longest list of every 16-row block
+    blocks = np.argsort(per_block)[-6:]
+    rows = np.unique(np.concatenate([np.arange(16 * b, 16 * b + 16) for b in blocks]
+                                    + [np.random.default_rng(1).choice(M, 160, replace=False)]))
+    B = spmm.synth_activations(N, K, seed=30)
+    s = spmm.HeteroSparse_SuggestSplitK(M, N, K)
+    C = run_fused(spmm, packed, words, offs, longest, B, M, N, K, s)
+    assert_close(C[:, rows], oracle.gemm_f32(np.ascontiguousarray(A[rows]), B))
+    items, offsets = spmm.InitSparseMatrixA_API(A2)
+    two = run_hybrid(spmm, packed, items, offsets, B, M, N, K, s, spmm.SpMM_SuggestSplitK(M, N, K))
+    diff = np.abs(C.astype(np.float32) - two.astype(np.float32))
+    assert np.isfinite(C).all() and (diff <= 2e-2 + 2e-2 * np.abs(two.astype(np.float32))).all()
