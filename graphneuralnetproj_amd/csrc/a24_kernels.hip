@@ -289,7 +289,7 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
     // this thread's chunks of the activation tile: token c / 16, columns (c % 16) * 8 .. + 8
     // (RM: chunk c of the unit's contiguous block, i.e. tokens 8 (c % (n_tokens / 8)) .. + 7 of row
     // c / (n_tokens / 8), kept where it sits in memory)
-    auto rm_byte = [&](int k, int n) {  // LDS byte of B[unit's row k][token n], RM only
+    auto rm_byte = [&](int k, int n) __attribute__((always_inline)) {  // LDS byte of B[unit's row k][token n], RM only
         return n_tokens == 64 ? k * 128 + ((((n >> 4) ^ (k >> 1)) & 3) << 5) + (n & 15) * 2 : (k * n_tokens + n) * 2;
     };
     const _Float16* src[CH];
@@ -333,7 +333,7 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
         tr_lane[0] = NT == 4 ? base0 + 32 * (l15 >> 3) : base0;
         tr_lane[1] = NT == 4 ? base0 + 32 - 32 * (l15 >> 3) : base0;
     }
-    auto tr_at = [&](int t, int hh) {
+    auto tr_at = [&](int t, int hh) __attribute__((always_inline)) {
         return NT == 4 ? tr_lane[t & 1] + 512 * hh + 64 * ((t >> 1) ^ hh) : tr_lane[0] + 4 * hh * rm_row_bytes + 32 * t;
     };
     const int tr_step = 32 * rm_row_bytes;
@@ -365,6 +365,41 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
     };
     constexpr int kLoadsA = (3 + RL) * RB;      // loads of one unit's records and lists per lane
     constexpr int kLoadsHead = RL > 0 ? 1 : 0;  // the offsets load that leads a unit's loads
+    // A launch with the most rounds (five, 320 words) may meet lists that are longer still (blocks
+    // of a row-skewed or nearly dense weight; a residual block holds up to 1024 words).  EX further
+    // rounds of such a list are fetched when the unit's turn comes, ahead of the loads that the
+    // same phase issues for the unit two further on, and awaited with the count of just those
+    // loads; whatever a list holds beyond that comes through ordinary loads inside the
+    // multiplication, which wait for everything in flight.  Extra loads never invalidate the
+    // constant waits elsewhere: a wait that allows N loads to stay outstanding covers the loads it
+    // is meant for however many younger ones there are.
+    constexpr bool kLong = RL == 5;
+    constexpr int EX = 3;
+    constexpr int kLoadsUnit = kLoadsHead + CH + kLoadsA;  // what issue_unit puts in flight
+    unsigned ex[RB][EX] = {};
+    auto any_longer = [&](const UnitRegs& x) __attribute__((always_inline)) {
+        bool any = false;
+#pragma unroll
+        for (int r = 0; r < RB; r++)
+            any = any || x.count[r] > RL * kWave;
+        return any;
+    };
+    auto issue_extras = [&](const UnitRegs& x) __attribute__((always_inline)) {
+        if constexpr (kLong) {
+            if (any_longer(x)) {  // all RB * EX loads or none: lanes and rounds past a list's end repeat its last word
+#pragma unroll
+                for (int r = 0; r < RB; r++) {
+                    const int last = x.count[r] > 0 ? x.count[r] - 1 : 0;
+#pragma unroll
+                    for (int i = 0; i < EX; i++) {
+                        const int at = lane + (RL + i) * kWave;
+                        const unsigned* p = words + x.start[r] + (at < last ? at : last);
+                        asm volatile("global_load_dword %0, %1, off nt" : "=v"(ex[r][i]) : "v"(p));
+                    }
+                }
+            }
+        }
+    };
     // lists are numbered like records: this wave's RB lists of a unit are neighbours
     const long list0 = ((long)(block0 / kGroupBlocks) * units) * kGroupBlocks + block0 % kGroupBlocks;
     const int* const off_lane = offsets + list0 + (lane <= RB ? lane : RB);
@@ -372,7 +407,7 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
     // A unit's loads: the offsets of the unit after it, its activation chunks (needed first), its
     // records, and (issue_words; o[0..RB] = the offsets of the unit's lists, the same in every lane)
     // its residual words.
-    auto issue_head = [&](UnitRegs& x, int unit, int unit_after) {
+    auto issue_head = [&](UnitRegs& x, int unit, int unit_after) __attribute__((always_inline)) {
         if constexpr (RL > 0)
             asm volatile("global_load_dword %0, %1, off" : "=v"(x.next) : "v"(off_lane + (size_t)unit_after * kGroupBlocks));
 #pragma unroll
@@ -382,7 +417,7 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
         for (int r = 0; r < RB; r++)
             x.a[r] = issue_a(rec[r] + (size_t)unit * kUnitStride + lane * 16, rec[r] + (size_t)unit * kUnitStride + lane * 4);
     };
-    auto issue_words = [&](UnitRegs& x, const int (&o)[RB + 1]) {
+    auto issue_words = [&](UnitRegs& x, const int (&o)[RB + 1]) __attribute__((always_inline)) {
         if constexpr (RL > 0) {
 #pragma unroll
             for (int r = 0; r < RB; r++) {
@@ -399,12 +434,12 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
             }
         }
     };
-    auto issue_unit = [&](UnitRegs& x, int unit, int unit_after, const int (&o)[RB + 1]) {
+    auto issue_unit = [&](UnitRegs& x, int unit, int unit_after, const int (&o)[RB + 1]) __attribute__((always_inline)) {
         issue_head(x, unit, unit_after);
         issue_words(x, o);
     };
     // The offsets that a unit's `next` load brought, once it has landed.
-    auto offsets_from = [&](UnitRegs& x, int (&o)[RB + 1]) {
+    auto offsets_from = [&](UnitRegs& x, int (&o)[RB + 1]) __attribute__((always_inline)) {
         if constexpr (RL > 0) {
             settle(x.next);
 #pragma unroll
@@ -412,14 +447,14 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
                 o[j] = __builtin_amdgcn_readlane(x.next, j);
         }
     };
-    auto store_b = [&](UnitRegs& x, int buf) {
+    auto store_b = [&](UnitRegs& x, int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < CH; i++) {
             settle(x.stage[i]);
             *reinterpret_cast<u32x4*>(tile + buf * kBuf + dst[i]) = x.stage[i];
         }
     };
-    auto landed = [&](UnitRegs& x) {
+    auto landed = [&](UnitRegs& x) __attribute__((always_inline)) {
 #pragma unroll
         for (int r = 0; r < RB; r++) {
             settle(x.a[r].v[0]);
@@ -434,9 +469,19 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
     };
     // where this lane's dense operands sit in the image: row lane % 16, granule (4 s + lane / 16) ^ row
     const int img_row = (lane & 15) * 256;
-    auto multiply_from = [&](UnitRegs& x, int buf) {
+    auto multiply_from = [&](UnitRegs& x, int buf) __attribute__((always_inline)) {
         const AFrag(&a)[RB] = x.a;
         half8 dense[RB][4];
+        if constexpr (kLong) {
+            if (any_longer(x)) {  // the extra rounds were issued just before this phase's issue_unit
+                wait_loads<kLoadsUnit>();
+#pragma unroll
+                for (int r = 0; r < RB; r++)
+#pragma unroll
+                    for (int i = 0; i < EX; i++)
+                        settle(ex[r][i]);
+            }
+        }
         if constexpr (RL > 0) {
             // One list after the other through the wave's image: LDS operations of a wave run in
             // order, so values, read-back and zeros need no barrier.
@@ -448,17 +493,29 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
                     for (int i = 0; i < RL; i++)
                         if (i == 0 || n > i * kWave)
                             *reinterpret_cast<unsigned short*>(image + (x.w[r][i] >> 16)) = static_cast<unsigned short>(x.w[r][i]);
-                    // A list longer than the RL rounds that travel with the unit (a block of a
-                    // row-skewed weight; a residual block holds up to 1024 words): the rest is fetched
-                    // here, with ordinary loads, which wait for everything this wave has in flight.
-                    // That stalls the wave's pipeline once per such list; the constant waits further
-                    // on stay right, since they only ever ask for fewer loads to be outstanding.
-                    const bool longer = n > RL * kWave;
-                    if (longer) {
-                        for (int at0 = RL * kWave; at0 < n; at0 += kWave) {
-                            const int at = at0 + lane;
-                            const unsigned w = words[x.start[r] + (at < n ? at : n - 1)];
-                            *reinterpret_cast<unsigned short*>(image + (w >> 16)) = static_cast<unsigned short>(w);
+                    // A list longer than the RL rounds that travel with the unit: EX more rounds
+                    // have just landed (above); the rest is fetched here, with ordinary loads,
+                    // which wait for everything this wave has in flight (a stall per round, for
+                    // lists of more than 512 words only).
+                    const bool longer = kLong && n > RL * kWave;
+                    if constexpr (kLong) {
+                        if (longer) {
+                            // (already waited for at the top on every real path: repeated here so
+                            // that wait and use sit under one condition, which is what the build's
+                            // checker of in-flight registers can follow)
+                            wait_loads<kLoadsUnit>();
+#pragma unroll
+                            for (int i = 0; i < EX; i++)
+                                settle(ex[r][i]);
+#pragma unroll
+                            for (int i = 0; i < EX; i++)
+                                if (n > (RL + i) * kWave)
+                                    *reinterpret_cast<unsigned short*>(image + (ex[r][i] >> 16)) = static_cast<unsigned short>(ex[r][i]);
+                            for (int at0 = (RL + EX) * kWave; at0 < n; at0 += kWave) {
+                                const int at = at0 + lane;
+                                const unsigned w = words[x.start[r] + (at < n ? at : n - 1)];
+                                *reinterpret_cast<unsigned short*>(image + (w >> 16)) = static_cast<unsigned short>(w);
+                            }
                         }
                     }
 #pragma unroll
@@ -524,7 +581,7 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
     int u = u0;  // every wave of the workgroup walks the same units: the barriers below are uniform
     if (u < u1) {
         const int last = u1 - 1;
-        auto ahead = [&](int d) { return u + d < last ? u + d : last; };
+        auto ahead = [&](int d) __attribute__((always_inline)) { return u + d < last ? u + d : last; };
         int o[RB + 1] = {};
         if constexpr (RL > 0) {
             // The first two units' offsets are fetched by themselves, and their records and
@@ -555,7 +612,7 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
         wait_loads<kLoadsA + kLoadsHead + CH + kLoadsA>();  // the first tile
         store_b(x[0], 0);
         __syncthreads();
-        auto phase = [&](auto kc, auto is_first) {  // unit u, whose registers are set kc
+        auto phase = [&](auto kc, auto is_first) __attribute__((always_inline)) {  // unit u, whose registers are set kc
             constexpr int k = decltype(kc)::value;
             const int buf = (u - u0) & 1;
             if constexpr (RL > 0 && decltype(is_first)::value)
@@ -563,6 +620,7 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
             else
                 wait_loads<kLoadsA>();
             landed(x[k]);
+            issue_extras(x[k]);
             store_b(x[(k + 1) % 3], buf ^ 1);
             int o2[RB + 1] = {};
             offsets_from(x[(k + 1) % 3], o2);  // unit u + 1 brought the offsets of unit u + 2
@@ -599,6 +657,11 @@ __global__ __launch_bounds__(W* kWave) void a24_spmm_shared_b_kernel(const uint8
             if constexpr (RL > 0)
                 settle(x[k].next);
         }
+#pragma unroll
+        for (int r = 0; r < RB; r++)
+#pragma unroll
+            for (int i = 0; i < EX; i++)
+                settle(ex[r][i]);
     }
 
     _Float16* dstc = out + (size_t)batch * slab;
