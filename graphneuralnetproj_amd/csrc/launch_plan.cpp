@@ -32,8 +32,8 @@ constexpr double kRoundUs = 4.00;           // start-up and drain of one round o
 constexpr double kNorm = 3.30;              // exponent that blends the three bounds
 constexpr double kCrowdPenalty = 0.043;     // per resident wave above kCrowdWaves on a unit
 constexpr double kCrowdWaves = 6.64;
-constexpr double kGlobalBPenalty = -0.01;  // mode 0, N <= 16, slice not staged: fragments from the L2 measure 1 to 1.5 %
-                                           // faster than the staged slice at the same shape (and fit where it does not)
+constexpr double kGlobalBPenalty = 0.0;    // mode 0, N <= 16, slice not staged: fragments from the L2 measure 1 to 1.5 % faster
+                                           // than the staged slice at the same shape; priced alike, and tried first
 constexpr double kModeKPenalty = 0.020;     // mode 1: activations from L2, reduction in LDS
 constexpr double kReduceUs = 3.44;          // fixed cost of the reduction as a second kernel (mode 0)
 constexpr double kFusedReduceUs = 2.19;     // ... and inside the main kernel (mode 1)
@@ -214,9 +214,10 @@ LaunchPlan plan_launch(int M, int N, int K, int split_k, bool row_major, double*
                 if (mode == 1 && w != 4)
                     continue;
                 // The row-sharing layout is only considered in the shapes the tuner measures and
-                // the constants were fitted on: 5..8 waves up to 16 tokens (the batch's activation
-                // slice staged in LDS or, what wins wherever both fit, its fragments from the
-                // L2), fragments from memory and 1, 2 or 4 waves above.
+                // the constants were fitted on: 5..8 waves up to 16 tokens, the batch's activation
+                // slice staged in LDS or, tried first and kept at equal cost because it measures a
+                // little faster wherever both fit, its fragments from the L2; fragments from memory
+                // and 1, 2 or 4 waves above.
                 if (mode == 0 && (N <= 16 ? w < 5 : (stage || (w != 1 && w != 2 && w != 4))))
                     continue;
                 LaunchPlan p{mode, w, row_major ? 0 : stage, 0};
