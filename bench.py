@@ -62,13 +62,13 @@ MEASURED_TRAFFIC_BYTES = {
     ("opt30b_ffn1", 16, 8, 0.8): (175.50e6, "profiles/tcsl_spmm_kernel_opt30b_ffn1_n16_pmc.txt"),  # mode 0: plus 7.34 MB of partial sums
     ("opt30b_ffn1", 64, 1, 0.8): (177.52e6, "profiles/tcsl_spmm_kernel_sweep_cases_hbm_traffic.txt"),
     ("opt30b_ffn1", 32, 1, 0.8): (171.70e6, "profiles/tcsl_spmm_kernel_sweep_cases_hbm_traffic.txt"),
-    ("opt30b_ffn1", 8, 1, 0.8): (167.50e6, "profiles/tcsl_spmm_kernel_sweep_cases_hbm_traffic.txt"),
+    ("opt30b_ffn1", 8, 1, 0.8): (167.29e6, "profiles/tcsl_spmm_kernel_sweep_cases_hbm_traffic.txt"),
     ("opt30b_ffn1", 16, 1, 0.9): (86.15e6, "profiles/tcsl_spmm_kernel_sweep_cases_hbm_traffic.txt"),
     ("opt30b_ffn1", 16, 1, 0.7): (251.38e6, "profiles/tcsl_spmm_kernel_sweep_cases_hbm_traffic.txt"),
     ("opt30b_ffn2", 16, 4, 0.8): (174.77e6, "profiles/tcsl_spmm_kernel_sweep_cases_hbm_traffic.txt"),
     ("opt30b_outproj", 16, 4, 0.8): (44.78e6, "profiles/tcsl_spmm_kernel_sweep_cases_hbm_traffic.txt"),
-    ("opt30b_qkv", 16, 8, 0.8): (132.08e6, "profiles/tcsl_spmm_kernel_sweep_cases_hbm_traffic.txt"),
-    ("opt66b_ffn1", 16, 6, 0.8): (284.90e6, "profiles/tcsl_spmm_kernel_sweep_cases_hbm_traffic.txt"),
+    ("opt30b_qkv", 16, 8, 0.8): (132.20e6, "profiles/tcsl_spmm_kernel_sweep_cases_hbm_traffic.txt"),
+    ("opt66b_ffn1", 16, 6, 0.8): (285.10e6, "profiles/tcsl_spmm_kernel_sweep_cases_hbm_traffic.txt"),
 }
 TRAFFIC_SOURCE = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, scaled by a copy kernel of known "
                   "size; summary in the named profile (not measured live)")
