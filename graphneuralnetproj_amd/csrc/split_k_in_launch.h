@@ -7,6 +7,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace inlaunch {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -72,36 +74,73 @@ __device__ __forceinline__ void fused_reduction_tail(const _Float16* __restrict_
     relu &= 0xff;
     nrows = nrows < M - row0 ? nrows : M - row0;
     const int per_tok = nrows / 8;
+    const int total = per_tok * N;  // runs of eight rows to sum
     const size_t slab = (size_t)M * N;
-    for (int c = threadIdx.x; c < per_tok * N; c += nthreads) {
-        const int tok = c / per_tok, m8 = c - tok * per_tok;
-        const size_t at = row_major ? (size_t)row0 * N + (size_t)c * 8 : (size_t)tok * M + row0 + m8 * 8;
-        const _Float16* w0 = slabs + at;
-        float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        int sidx = 0;
-        for (; sidx + 4 <= split_k; sidx += 4) {
-            half8 w[4];
+    // Every load is served from memory, and a thread can only add what has arrived.  A thread with
+    // several runs of eight rows (64 tokens: four per thread) keeps four slabs of four runs in flight,
+    // sixteen 16-byte loads, so that its trips to memory are ceil(split_k / 4) in all rather than per
+    // run (9216 x 9216, 64 tokens, three batches: 28.9 -> 26.2 us).  Each element's slabs are still
+    // added in slab order.  (Sixteen slabs of one run at a time, for the threads that have a single
+    // run, measured 2 to 3 % slower than four even where there are only four.)
+    auto sum_runs = [&](auto it_c, auto g_c) __attribute__((always_inline)) {
+        constexpr int IT = decltype(it_c)::value, G = decltype(g_c)::value;
+        for (int c0 = threadIdx.x; c0 < total; c0 += nthreads * IT) {
+            size_t at[IT];
+            float sum[IT][8];
 #pragma unroll
-            for (int u = 0; u < 4; u++)
-                w[u] = load_through(w0 + (size_t)(sidx + u) * slab);
-#pragma unroll
-            for (int u = 0; u < 4; u++)
+            for (int i = 0; i < IT; i++) {
+                const int c = c0 + i * nthreads < total ? c0 + i * nthreads : c0;  // a run past the end repeats the first
+                const int tok = c / per_tok, m8 = c - tok * per_tok;
+                at[i] = row_major ? (size_t)row0 * N + (size_t)c * 8 : (size_t)tok * M + row0 + m8 * 8;
 #pragma unroll
                 for (int j = 0; j < 8; j++)
-                    sum[j] += static_cast<float>(w[u][j]);
-        }
-        for (; sidx < split_k; sidx++) {
-            const half8 w = load_through(w0 + (size_t)sidx * slab);
+                    sum[i][j] = 0.f;
+            }
+            int sidx = 0;
+            for (; sidx + G <= split_k; sidx += G) {
+                half8 w[IT][G];
 #pragma unroll
-            for (int j = 0; j < 8; j++)
-                sum[j] += static_cast<float>(w[j]);
-        }
-        half8 o;
+                for (int u = 0; u < G; u++)
 #pragma unroll
-        for (int j = 0; j < 8; j++)
-            o[j] = static_cast<_Float16>(relu ? fmaxf(sum[j], 0.f) : sum[j]);
-        *reinterpret_cast<half8*>(C + (row_major ? at : (size_t)tok * ldc + row0 + m8 * 8)) = o;
-    }
+                    for (int i = 0; i < IT; i++)
+                        w[i][u] = load_through(slabs + at[i] + (size_t)(sidx + u) * slab);
+#pragma unroll
+                for (int u = 0; u < G; u++)
+#pragma unroll
+                    for (int i = 0; i < IT; i++)
+#pragma unroll
+                        for (int j = 0; j < 8; j++)
+                            sum[i][j] += static_cast<float>(w[i][u][j]);
+            }
+            for (; sidx < split_k; sidx++) {
+                half8 w[IT];
+#pragma unroll
+                for (int i = 0; i < IT; i++)
+                    w[i] = load_through(slabs + at[i] + (size_t)sidx * slab);
+#pragma unroll
+                for (int i = 0; i < IT; i++)
+#pragma unroll
+                    for (int j = 0; j < 8; j++)
+                        sum[i][j] += static_cast<float>(w[i][j]);
+            }
+#pragma unroll
+            for (int i = 0; i < IT; i++) {
+                const int c = c0 + i * nthreads;
+                if (c >= total)
+                    break;
+                half8 o;
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    o[j] = static_cast<_Float16>(relu ? fmaxf(sum[i][j], 0.f) : sum[i][j]);
+                const int tok = c / per_tok, m8 = c - tok * per_tok;
+                *reinterpret_cast<half8*>(C + (row_major ? at[i] : (size_t)tok * ldc + row0 + m8 * 8)) = o;
+            }
+        }
+    };
+    if (total <= nthreads)
+        sum_runs(std::integral_constant<int, 1>{}, std::integral_constant<int, 4>{});
+    else
+        sum_runs(std::integral_constant<int, 4>{}, std::integral_constant<int, 4>{});
     if (threadIdx.x == 0)
         *counter = 0;  // ready for the next call
 }
