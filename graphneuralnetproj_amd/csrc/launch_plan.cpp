@@ -23,7 +23,8 @@ constexpr int kCUs = 256;
 
 // Fitted constants (microseconds, bytes per microsecond): least squares on the logarithm of
 // estimate / measurement over every plan within 30 % of its shape's best in the tuner's logs
-// (24 shapes x 4 token counts at 80 % sparsity, 3245 points), checked on ten shapes the fit never saw.
+// (24 shapes x 4 token counts at 80 % sparsity, 3245 points; the two constants of the in-launch sum
+// also on ten small matrices of 8 to 96 tile rows), checked on ten shapes the fit never saw.
 constexpr double kLaunchUs = 3.16;          // fixed cost of the main kernel
 constexpr double kTileBytes = kTileBytesAt80;  // one tile at 80 % sparsity: what the constants below were fitted on
 constexpr double kChipBytesPerUs = 9.92e6;  // whole-chip stream rate
@@ -37,8 +38,9 @@ constexpr double kCrowdPenalty = 0.0436;    // per resident wave above kCrowdWav
 constexpr double kCrowdWaves = 4.0;
 constexpr double kModeKPenalty = 0.0626;    // mode 1: no sharing of fragments, reduction in LDS
 constexpr double kReduceUs = 2.48;          // fixed cost of the reduction as a second kernel (mode 0)
-constexpr double kFusedReduceUs = 0.949;    // ... and inside the main kernel (mode 1)
+constexpr double kFusedReduceUs = 0.494;    // ... and inside the main kernel (mode 1)
 constexpr double kReduceBytesPerUs = 5.375e6;
+constexpr double kFusedWgBytesPerUs = 33.0e3;  // ... where the last workgroup of a tile row pulls Split_K slabs of 128 x N values alone
 
 int column_blocks(int N)
 {
@@ -194,8 +196,11 @@ double plan_cost_us(int M, int N, int K, int split_k, const LaunchPlan& p, doubl
     }
     if (p.mode == 1)
         total *= 1.0 + kModeKPenalty;
-    if (split_k > 1)
+    if (split_k > 1) {
         total += (p.mode == 1 ? kFusedReduceUs : kReduceUs) + (2.0 * split_k + 1.0) * M * N * 2.0 / kReduceBytesPerUs;
+        if (p.mode == 1)
+            total += static_cast<double>(split_k) * N * (kTileRows * 2) / kFusedWgBytesPerUs;
+    }
     return total;
 }
 
