@@ -56,7 +56,10 @@ int max_waves(int N)
 // stage_b}: one table per sparsity the benchmark names.  A caller that knows the weight's bytes
 // gets its Split_K from the table of the nearest density; a call, which knows only (M, N, K,
 // Split_K), takes the launch shape of whichever table holds that Split_K for the shape (80 %
-// first), so the Split_K that a converter stored carries the choice to the run.
+// first), so the Split_K that a converter stored carries the choice to the run.  A shape's first
+// row is its measured best; further rows of the same (M, K, N) hold the best launch shape for
+// other Split_K values a caller may fix (the benchmark's sweep of 1, 2, 4, 7 on the attention
+// projections; tune_plans.py --split-k).
 struct Tuned {
     int M, K, N, split_k, mode, waves, stage_b;
 };

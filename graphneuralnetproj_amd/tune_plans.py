@@ -23,8 +23,22 @@ OPT_SHAPES = ("28672x7168,7168x28672,21504x7168,7168x7168,27648x9216,9216x9216,3
               "13824x9216,9216x4608,18432x9216,9216x18432,6912x9216,9216x2304")  # ... and of OPT-66B
 
 
-def candidate_plans(N, tiles_k):
+def candidate_plans(N, tiles_k, only=None):
+    """The grid of (Split_K, mode, waves, stage_b); only = the Split_K values to keep (then every launch
+    shape of the grid is tried with each of them, also those the full grid skips for that Split_K)."""
     max_w = 8 if N <= 32 else 4
+    if only:
+        plans = []
+        for S in only:
+            if S > tiles_k or (S > 1 and -(-tiles_k // S) * (S - 1) >= tiles_k):
+                continue  # a batch would be empty
+            plans += [(S, 1, w, 0) for w in range(3, max_w + 1)]
+            if N <= 16:
+                plans += [(S, 0, w, st) for w in (5, 6, 7, 8) for st in (1, 0)]
+            else:
+                plans += [(S, 0, w, 0) for w in ((1, 2, 3, 4, 5, 6, 8) if N == 32 else (1, 2, 3, 4))]
+                plans += [(S, 0, w, 2) for w in ((4, 8) if N == 32 else (4,))]
+        return plans
     plans = []
     for S in (1, 2, 3, 4, 6, 8, 12, 16, 24, 32):
         if S <= tiles_k:
@@ -49,6 +63,9 @@ def main():
     ap.add_argument("--tokens", default="8,16,32,64")
     ap.add_argument("--sparsity", type=float, default=0.8)
     ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--split-k", default=None,
+                    help="comma-separated Split_K values: one row per (shape, N, Split_K) with the best launch shape "
+                         "for that Split_K (rows to append after the shape's own best, for callers that fix Split_K)")
     ap.add_argument("--out", default=None, help="write the table rows here (default: stdout only)")
     ap.add_argument("--log", default=None, help="write every measurement as JSON lines here")
     args = ap.parse_args()
@@ -90,7 +107,8 @@ def main():
             want = d_C.float().clone()
             tol = 2e-2 + 2e-2 * want.abs()
             results = []
-            for plan in candidate_plans(N, K // 64):
+            only = [int(x) for x in args.split_k.split(",")] if args.split_k else None
+            for plan in candidate_plans(N, K // 64, only):
                 if call(0, plan) != 0:
                     continue  # does not fit
                 torch.cuda.synchronize()
@@ -106,9 +124,17 @@ def main():
                 torch.cuda.synchronize()
                 results.append(((time.perf_counter() - t0) / args.steps * 1e6, plan))
             results.sort()
-            us, (S, mode, w, st) = results[0]
-            rows.append(f"    {{{M}, {K}, {N}, {S}, {mode}, {w}, {st}}},  // {us:.1f} us")
-            print(rows[-1], "   runners-up:", "  ".join(f"{p}: {u:.1f}" for u, p in results[1:4]), flush=True)
+            if only:
+                for S in only:
+                    per = [r for r in results if r[1][0] == S]
+                    if per:
+                        us, (_, mode, w, st) = per[0]
+                        rows.append(f"    {{{M}, {K}, {N}, {S}, {mode}, {w}, {st}}},  // {us:.1f} us")
+                        print(rows[-1], "   runners-up:", "  ".join(f"{p}: {u:.1f}" for u, p in per[1:4]), flush=True)
+            else:
+                us, (S, mode, w, st) = results[0]
+                rows.append(f"    {{{M}, {K}, {N}, {S}, {mode}, {w}, {st}}},  // {us:.1f} us")
+                print(rows[-1], "   runners-up:", "  ".join(f"{p}: {u:.1f}" for u, p in results[1:4]), flush=True)
             if log:
                 log.write(json.dumps({"M": M, "K": K, "N": N, "a_bytes": a_bytes,
                                       "results": [[u, *p] for u, p in results]}) + "\n")
