@@ -43,7 +43,7 @@ def candidate_plans(N, tiles_k, only=None):
     for S in (1, 2, 3, 4, 6, 8, 12, 16, 24, 32):
         if S <= tiles_k:
             plans += [(S, 1, w, 0) for w in range(3, max_w + 1)]
-    for S in (4, 6, 7, 8, 10, 12, 14, 16, 20, 24, 28, 32):
+    for S in (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 14, 16, 20, 24, 28, 32):
         if S <= tiles_k and N <= 16:
             plans += [(S, 0, w, 1) for w in (5, 6, 7, 8)]
             plans += [(S, 0, w, 0) for w in (6, 7, 8)]  # the slice not staged (what fits when it would not): fragments from the L2
