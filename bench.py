@@ -232,7 +232,8 @@ def sweep_cases():
                 cases.append((f"{name}_n{N}_split{split_k}", f"opt30b_{name}", N, 0.8, False, split_k))
     for model in ("opt66b", "opt175b"):
         for name in ("qkv", "outproj", "ffn1", "ffn2"):
-            for N in (16, 8, 32):
+            # 64 tokens where the matrix has 288 and more tile rows (few batches of row-sharing workgroups)
+            for N in (16, 8, 32) + ((64,) if (model, name) in (("opt66b", "ffn1"), ("opt175b", "qkv"), ("opt175b", "ffn1")) else ()):
                 cases.append((f"{model}_{name}" if N == 16 else f"{model}_{name}_n{N}", f"{model}_{name}", N, 0.8, False, 0))
     return cases
 
