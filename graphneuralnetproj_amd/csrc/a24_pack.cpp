@@ -240,7 +240,8 @@ int pack_residual(const uint16_t* A2, int M, int K, uint32_t** words, int** offs
                             list.push_back(row[c] | residual_address(r, c) << 16);
                 }
                 order_by_bank(list, tmp);
-                std::memcpy(out + off[record_index(rb, u, units)], list.data(), list.size() * sizeof(uint32_t));
+                if (!list.empty())  // (an empty vector's data() may be null, which memcpy must not be given)
+                    std::memcpy(out + off[record_index(rb, u, units)], list.data(), list.size() * sizeof(uint32_t));
             }
     });
     *words = out;
