@@ -29,3 +29,23 @@ def test_host_code_is_clean_under_asan_and_ubsan(tmp_path):
     assert run.returncode == 0, (run.stdout[-2000:], run.stderr[-4000:])
     assert "clean, 0 failed checks" in run.stdout
     assert "runtime error" not in run.stderr and "AddressSanitizer" not in run.stderr
+
+
+def test_counter_pages_are_race_free_under_tsan(tmp_path):
+    """The pages of arrival counters handed out from sixteen host threads at once (own streams, the
+    per-thread default stream, short-lived streams that force pages to change hands, captures), in a
+    ThreadSanitizer build: no data race, and no page given to a caller while another caller's launch
+    on it is still in flight (tests/support/counter_pages_threads.cpp)."""
+    if shutil.which("g++") is None:
+        pytest.skip("no g++")
+    exe = tmp_path / "cp_threads"
+    build = subprocess.run(
+        ["g++", "-std=c++17", "-O1", "-g", "-fsanitize=thread", "-pthread", "-I", CSRC, "-o", str(exe),
+         os.path.join(ROOT, "tests", "support", "counter_pages_threads.cpp"), os.path.join(CSRC, "counter_pages.cpp")],
+        capture_output=True, text=True)
+    assert build.returncode == 0, build.stderr[-2000:]
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300)
+    if "unexpected memory mapping" in run.stderr:
+        pytest.skip("ThreadSanitizer cannot map its shadow memory on this kernel")
+    assert run.returncode == 0, (run.stdout[-2000:], run.stderr[-4000:])
+    assert "violations 0" in run.stdout and "ThreadSanitizer" not in run.stderr
