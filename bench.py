@@ -314,6 +314,8 @@ def sweep(G, lib, torch, dev, sptr, with_stack):
                     "split_k_from": "sweep" if forced_split else "planner",
                     "layout": "B[K][N], C[M][N]" if row_major else "B[N][K], C[N][M]",
                     "plan": f"mode {plan['mode']}, {plan['waves']} waves", "compressed_bytes": a_bytes,
+                    "reduction": ("none" if split_k == 1 else
+                                  "in launch" if G.SpMM_PlanReductionInLaunch(M, N, K, split_k) else "kernel"),
                     "ms": ms, "frac": a_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                     "kernel_ms": kernel_ms,
                     "kernel_frac": a_bytes / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS if kernel_ms else None,

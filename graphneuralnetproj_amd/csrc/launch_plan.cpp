@@ -23,24 +23,26 @@ constexpr int kCUs = 256;
 
 // Fitted constants (microseconds, bytes per microsecond): least squares on the logarithm of
 // estimate / measurement over every plan within 30 % of its shape's best in the tuner's logs
-// (24 shapes x 4 token counts at 80 % sparsity, 3245 points; the two constants of the in-launch sum
-// also on ten small matrices of 8 to 96 tile rows), checked on ten shapes the fit never saw.
-constexpr double kLaunchUs = 3.16;          // fixed cost of the main kernel
+// (24 shapes x 4 token counts at 80 % sparsity) and over the same grid, with the reduction kernel behind
+// the K-splitting launches as well, on ten small matrices of 8 to 96 tile rows (4632 points in all),
+// checked on ten shapes the fit never saw.
+constexpr double kLaunchUs = 2.985;         // fixed cost of the main kernel
 constexpr double kTileBytes = kTileBytesAt80;  // one tile at 80 % sparsity: what the constants below were fitted on
-constexpr double kChipBytesPerUs = 9.92e6;  // whole-chip stream rate
-constexpr double kCuBytesPerUs = 75.6e3;    // what one compute unit's vector memory path can pull
-constexpr double kFragWeight = 0.656;        // weight of a tile's activation fragments (2 KiB per 16 tokens) on that path ...
-constexpr double kFragUnshared = 0.435;     // ... of which the row-sharing waves of a workgroup share the rest through the L1
-constexpr double kMfmaTileUs = 0.184;       // serial MFMA + LDS time per tile and 16-token block
-constexpr double kRoundUs = 3.00;           // start-up and drain of one round of workgroups
-constexpr double kNorm = 1.404;             // exponent that blends the three bounds (close to a sum)
-constexpr double kCrowdPenalty = 0.0436;    // per resident wave above kCrowdWaves on a unit
+constexpr double kChipBytesPerUs = 10.95e6; // whole-chip stream rate
+constexpr double kCuBytesPerUs = 65.79e3;   // what one compute unit's vector memory path can pull
+constexpr double kFragWeight = 0.494;       // weight of a tile's activation fragments (2 KiB per 16 tokens) on that path ...
+constexpr double kFragUnshared = 0.284;     // ... of which the row-sharing waves of a workgroup share the rest through the L1
+constexpr double kMfmaTileUs = 0.201;       // serial MFMA + LDS time per tile and 16-token block
+constexpr double kRoundUs = 2.885;          // start-up and drain of one round of workgroups
+constexpr double kNorm = 1.386;             // exponent that blends the three bounds (close to a sum)
+constexpr double kCrowdPenalty = 0.0593;    // per resident wave above kCrowdWaves on a unit
 constexpr double kCrowdWaves = 4.0;
-constexpr double kModeKPenalty = 0.0626;    // mode 1: no sharing of fragments, reduction in LDS
-constexpr double kReduceUs = 2.48;          // fixed cost of the reduction as a second kernel (mode 0)
-constexpr double kFusedReduceUs = 0.494;    // ... and inside the main kernel (mode 1)
-constexpr double kReduceBytesPerUs = 5.375e6;
-constexpr double kFusedWgBytesPerUs = 33.0e3;  // ... where the last workgroup of a tile row pulls Split_K slabs of 128 x N values alone
+constexpr double kModeKPenalty = 0.0474;    // mode 1: no sharing of fragments, reduction in LDS
+constexpr double kReduceUs = 2.566;         // fixed cost of the reduction as a second kernel
+constexpr double kFusedReduceUs = 0.712;    // ... and inside the main kernel (mode 1), where the last workgroup of a
+constexpr double kFusedSlabUs = 0.028;      //     tile row pulls Split_K slabs of 128 x N values alone: a term per slab
+constexpr double kFusedSlabTokenUs = 0.00694;  //  and one per slab and token
+constexpr double kReduceBytesPerUs = 5.989e6;
 
 int column_blocks(int N)
 {
@@ -62,6 +64,7 @@ int max_waves(int N)
 // projections; tune_plans.py --split-k).
 struct Tuned {
     int M, K, N, split_k, mode, waves, stage_b;
+    int separate_reduction = 0;  // an eighth value in a row: mode 1 with the reduction kernel
 };
 constexpr Tuned kTuned80[] = {
 #include "tuned_plans.inc"
@@ -200,9 +203,9 @@ double plan_cost_us(int M, int N, int K, int split_k, const LaunchPlan& p, doubl
     if (p.mode == 1)
         total *= 1.0 + kModeKPenalty;
     if (split_k > 1) {
-        total += (p.mode == 1 ? kFusedReduceUs : kReduceUs) + (2.0 * split_k + 1.0) * M * N * 2.0 / kReduceBytesPerUs;
-        if (p.mode == 1)
-            total += static_cast<double>(split_k) * N * (kTileRows * 2) / kFusedWgBytesPerUs;
+        const bool in_launch = p.mode == 1 && !p.separate_reduction;
+        total += (in_launch ? kFusedReduceUs + split_k * (kFusedSlabUs + kFusedSlabTokenUs * N) : kReduceUs) +
+                 (2.0 * split_k + 1.0) * M * N * 2.0 / kReduceBytesPerUs;
     }
     return total;
 }
@@ -214,6 +217,7 @@ LaunchPlan plan_launch(int M, int N, int K, int split_k, bool row_major, double*
         // (row-major activations are not staged per batch: every wave keeps its own tile of them in
         // LDS, and the row-sharing shapes measure as fast that way as the staged column-major ones)
         LaunchPlan p{t->mode, t->waves, row_major ? 0 : t->stage_b, 0};
+        p.separate_reduction = t->separate_reduction != 0;
         if (complete_plan(N, K, split_k, row_major, p)) {
             if (cost_us)
                 *cost_us = plan_cost_us(M, N, K, split_k, p, tile_bytes);
@@ -233,17 +237,22 @@ LaunchPlan plan_launch(int M, int N, int K, int split_k, bool row_major, double*
                 // The row-sharing layout is only considered in the shapes the tuner measures and
                 // the constants were fitted on: 5..8 waves up to 16 tokens, the batch's activation
                 // slice staged in LDS or its fragments from the L2 (tried first); fragments from
-                // the L2 above, with 4 or 5 waves at 32 tokens and 1 to 4 at 64 (the model ranks the
-                // other wave counts of 32 tokens worse than they measure).
-                if (mode == 0 && (N <= 16 ? w < 5 : (stage || (N == 32 && w != 4 && w != 5))))
+                // the L2 above, with 4 waves at 32 tokens and 1 to 4 at 64 (the model cannot rank the
+                // other wave counts of 32 tokens: with them allowed it picks worse).
+                if (mode == 0 && (N <= 16 ? w < 5 : (stage || (N == 32 && w != 4))))
                     continue;
                 LaunchPlan p{mode, w, row_major ? 0 : stage, 0};
                 if (!complete_plan(N, K, split_k, row_major, p))
                     continue;
-                const double c = plan_cost_us(M, N, K, split_k, p, tile_bytes);
-                if (best_cost < 0 || c < best_cost) {
-                    best = p;
-                    best_cost = c;
+                // the K-splitting layout adds its slabs up inside the launch or leaves them to the
+                // reduction kernel, whichever the model prices lower (many batches, many tokens: the kernel)
+                for (int separate = 0; separate <= (mode == 1 && split_k > 1 ? 1 : 0); separate++) {
+                    p.separate_reduction = separate != 0;
+                    const double c = plan_cost_us(M, N, K, split_k, p, tile_bytes);
+                    if (best_cost < 0 || c < best_cost) {
+                        best = p;
+                        best_cost = c;
+                    }
                 }
             }
     if (cost_us)
@@ -255,6 +264,7 @@ int suggest_split_k(int M, int N, int K, LaunchPlan* plan, double tile_bytes)
 {
     if (const Tuned* t = find_tuned(M, N, K, 0, density_table(tile_bytes))) {
         LaunchPlan p{t->mode, t->waves, t->stage_b, 0};
+        p.separate_reduction = t->separate_reduction != 0;
         if (complete_plan(N, K, t->split_k, false, p)) {
             if (plan)
                 *plan = p;

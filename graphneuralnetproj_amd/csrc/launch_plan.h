@@ -7,11 +7,15 @@ namespace tcsl {
 //         batch (stage_b: the batch's activation slice is staged in LDS and shared);
 // mode 1: the W waves of a workgroup split the batch of one tile row among themselves and
 //         add their accumulators up in LDS.
+// separate_reduction (mode 1, Split_K > 1): the slabs of partial sums are added up by the reduction
+//         kernel instead of by the last workgroup of each tile row inside the launch (mode 0 always
+//         uses the reduction kernel).
 struct LaunchPlan {
     int mode;
     int waves;
     int stage_b;
     unsigned lds_bytes;
+    bool separate_reduction = false;
 };
 
 // True (and lds_bytes filled in) when the kernels can run this shape.

@@ -165,7 +165,7 @@ int launch_main(void* stream, const void* Compressed_A, const int* TileOffsets, 
     // A page from the pool stays this call's until the launch is enqueued (the lock): from then
     // on its stream counts as busy and the page cannot change hands.
     std::unique_lock<std::mutex> page_lock;
-    if (fused_out && p.mode == 1 && M / tcsl::kTileRows <= 4096) {
+    if (fused_out && p.mode == 1 && !p.separate_reduction && M / tcsl::kTileRows <= 4096) {
         if (o.static_workspace) {
             page = kStaticWorkspacePage;
         } else {
@@ -309,6 +309,17 @@ extern "C" int SpMM_PlanLaunch(int M, int N, int K, int Split_K, int* Mode, int*
     if (EstimatedUs)
         *EstimatedUs = cost;
     return 0;
+}
+
+extern "C" int SpMM_PlanReductionInLaunch(int M, int N, int K, int Split_K)
+{
+    if ((N != 8 && N != 16 && N != 32 && N != 64) || M <= 0 || K <= 0 || M % tcsl::kTileRows != 0 ||
+        K % tcsl::kTileCols != 0 || Split_K < 1)
+        return -1;
+    if (Split_K == 1)
+        return 0;
+    const tcsl::LaunchPlan p = tcsl::plan_launch(M, N, K, Split_K, false, nullptr);
+    return p.mode == 1 && !p.separate_reduction && M / tcsl::kTileRows <= 4096 ? 1 : 0;
 }
 
 extern "C" int SpMM_SplitK_API_Events(void* stream, const void* A, const void* Compressed_A, const int* TileOffsets,

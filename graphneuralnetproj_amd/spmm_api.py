@@ -38,6 +38,7 @@ EXPORTED_SYMBOLS = (
     "SpMM_SuggestSplitK",
     "SpMM_SuggestSplitK_Bytes",
     "SpMM_PlanLaunch",
+    "SpMM_PlanReductionInLaunch",
     "SpMM_SplitK_API_Planned",
     "SpMM_SplitK_API_RowMajor",
     "SpMM_SplitK_API_RowMajor_Flags",
@@ -135,6 +136,8 @@ def load_library():
     lib.SpMM_SuggestSplitK_Bytes.argtypes = [ctypes.c_int] * 3 + [ctypes.c_long]
     lib.SpMM_PlanLaunch.restype = ctypes.c_int
     lib.SpMM_PlanLaunch.argtypes = [ctypes.c_int] * 4 + [_i32p] * 4 + [ctypes.POINTER(ctypes.c_double)]
+    lib.SpMM_PlanReductionInLaunch.restype = ctypes.c_int
+    lib.SpMM_PlanReductionInLaunch.argtypes = [ctypes.c_int] * 4
     lib.SpMM_SplitK_API_Planned.restype = ctypes.c_int
     lib.SpMM_SplitK_API_Planned.argtypes = ([ctypes.c_void_p] * 5 + [ctypes.c_int] * 3 + [ctypes.c_void_p]
                                             + [ctypes.c_int] * 6)
@@ -384,6 +387,15 @@ def SpMM_PlanLaunch(M_Global, N_Global, K_Global, Split_K):
         raise SpMMError("SpMM_PlanLaunch", rc)
     return {"mode": vals[0].value, "waves": vals[1].value, "stage_b": vals[2].value, "lds_bytes": vals[3].value,
             "estimated_us": est.value}
+
+
+def SpMM_PlanReductionInLaunch(M_Global, N_Global, K_Global, Split_K):
+    """True if the planned call adds its slabs of partial sums up inside the main kernel's launch,
+    False if it runs the reduction kernel (or Split_K is 1)."""
+    rc = load_library().SpMM_PlanReductionInLaunch(M_Global, N_Global, K_Global, Split_K)
+    if rc < 0:
+        raise SpMMError("SpMM_PlanReductionInLaunch", rc)
+    return bool(rc)
 
 
 def SpMM_SplitK_API_RowMajor_Flags(stream, Compressed_A, TileOffsets, B, C, M_Global, N_Global, K_Global, Reduction_Workspace,

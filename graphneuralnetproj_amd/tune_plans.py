@@ -23,9 +23,31 @@ OPT_SHAPES = ("28672x7168,7168x28672,21504x7168,7168x7168,27648x9216,9216x9216,3
               "13824x9216,9216x4608,18432x9216,9216x18432,6912x9216,9216x2304")  # ... and of OPT-66B
 
 
+SEPARATE = 3  # in a plan tuple's last place with mode 1: the slabs are added up by the reduction kernel
+
+
+def planned_args(plan):
+    """(Split_K, Mode, Waves, StageB, Flags) of SpMM_SplitK_API_Planned for a plan tuple, launched as a planned call would be."""
+    from graphneuralnetproj_amd import SPMM_FLAG_ADAPTIVE_WAVES, SPMM_FLAG_SEPARATE_REDUCTION
+
+    S, mode, w, st = plan
+    if mode == 1 and st == SEPARATE:
+        return S, mode, w, 0, SPMM_FLAG_ADAPTIVE_WAVES | SPMM_FLAG_SEPARATE_REDUCTION
+    return S, mode, w, st, SPMM_FLAG_ADAPTIVE_WAVES
+
+
+def table_row(M, K, N, plan):
+    S, mode, w, st = plan
+    if mode == 1 and st == SEPARATE:
+        return f"{{{M}, {K}, {N}, {S}, {mode}, {w}, 0, 1}}"
+    return f"{{{M}, {K}, {N}, {S}, {mode}, {w}, {st}}}"
+
+
 def candidate_plans(N, tiles_k, only=None):
     """The grid of (Split_K, mode, waves, stage_b); only = the Split_K values to keep (then every launch
-    shape of the grid is tried with each of them, also those the full grid skips for that Split_K)."""
+    shape of the grid is tried with each of them, also those the full grid skips for that Split_K).
+    Mode 1 with more than one batch is tried with the sum inside the launch and, from four batches on and
+    with four waves, with the reduction kernel (last place SEPARATE)."""
     max_w = 8 if N <= 32 else 4
     if only:
         plans = []
@@ -33,6 +55,8 @@ def candidate_plans(N, tiles_k, only=None):
             if S > tiles_k or (S > 1 and -(-tiles_k // S) * (S - 1) >= tiles_k):
                 continue  # a batch would be empty
             plans += [(S, 1, w, 0) for w in range(3, max_w + 1)]
+            if S >= 4:
+                plans.append((S, 1, 4, SEPARATE))
             if N <= 16:
                 plans += [(S, 0, w, st) for w in (5, 6, 7, 8) for st in (1, 0)]
             else:
@@ -43,6 +67,8 @@ def candidate_plans(N, tiles_k, only=None):
     for S in (1, 2, 3, 4, 6, 8, 12, 16, 24, 32):
         if S <= tiles_k:
             plans += [(S, 1, w, 0) for w in range(3, max_w + 1)]
+            if S >= 4:
+                plans.append((S, 1, 4, SEPARATE))
     for S in (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 14, 16, 20, 24, 28, 32):
         if S <= tiles_k and N <= 16:
             plans += [(S, 0, w, 1) for w in (5, 6, 7, 8)]
@@ -96,10 +122,10 @@ def main():
             d_W = torch.zeros((32, N, M), dtype=torch.float16, device=dev)
 
             def call(i, plan):
-                S, mode, w, st = plan
+                S, mode, w, st, flags = planned_args(plan)
                 return lib.SpMM_SplitK_API_Planned(stream, d_items[i % copies].data_ptr(), d_offs.data_ptr(),
                                                    d_B.data_ptr(), d_C.data_ptr(), M, N, K, d_W.data_ptr(), S, mode, w, st, 0,
-                                                   G.SPMM_FLAG_ADAPTIVE_WAVES)  # as a planned call launches it
+                                                   flags)  # as a planned call launches it
 
             S0 = G.SpMM_SuggestSplitK(M, N, K)
             G.SpMM_SplitK_API(None, None, d_items[0], d_offs, d_B, d_C, M, N, K, d_W, S0)
@@ -129,11 +155,11 @@ def main():
                     per = [r for r in results if r[1][0] == S]
                     if per:
                         us, (_, mode, w, st) = per[0]
-                        rows.append(f"    {{{M}, {K}, {N}, {S}, {mode}, {w}, {st}}},  // {us:.1f} us")
+                        rows.append(f"    {table_row(M, K, N, (S, mode, w, st))},  // {us:.1f} us")
                         print(rows[-1], "   runners-up:", "  ".join(f"{p}: {u:.1f}" for u, p in per[1:4]), flush=True)
             else:
                 us, (S, mode, w, st) = results[0]
-                rows.append(f"    {{{M}, {K}, {N}, {S}, {mode}, {w}, {st}}},  // {us:.1f} us")
+                rows.append(f"    {table_row(M, K, N, (S, mode, w, st))},  // {us:.1f} us")
                 print(rows[-1], "   runners-up:", "  ".join(f"{p}: {u:.1f}" for u, p in results[1:4]), flush=True)
             if log:
                 log.write(json.dumps({"M": M, "K": K, "N": N, "a_bytes": a_bytes,
@@ -141,7 +167,8 @@ def main():
                 log.flush()
         del d_items
         torch.cuda.empty_cache()
-    text = ("// {M, K, N, Split_K, mode, waves, stage_b}  -- written by graphneuralnetproj_amd/tune_plans.py\n"
+    text = ("// {M, K, N, Split_K, mode, waves, stage_b[, 1 = mode 1 with the reduction kernel]}"
+            "  -- written by graphneuralnetproj_amd/tune_plans.py\n"
             + "\n".join(rows) + "\n")
     if args.out:
         with open(args.out, "w") as f:

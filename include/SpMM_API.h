@@ -266,6 +266,17 @@ SPMM_EXPORT int SpMM_PlanLaunch(int M_Global, int N_Global, int K_Global, int Sp
                                 int* LdsBytes, double* EstimatedUs);
 
 /*
+ * Where SpMM_SplitK_API adds the Split_K slabs of partial sums up for (M, N, K, Split_K): 1 = inside the
+ * main kernel's launch (Mode 1: the last workgroup to finish a tile row sums that row's slabs; what
+ * the planner picks for few batches), 0 = with the reduction kernel, the counterpart of the
+ * reference's SplitK_Reduction (csrc/Reduction_Kernel.cuh:24-47; Mode 0 always, Mode 1 with many
+ * batches or many tokens, where one workgroup pulling every slab of its rows costs more than a
+ * second kernel), or Split_K == 1.  Same bits either way.  -1 for a shape the kernels do not take.
+ * A call may still fall back to the reduction kernel (SPMM_FLAG_SEPARATE_REDUCTION, no free counters).
+ */
+SPMM_EXPORT int SpMM_PlanReductionInLaunch(int M_Global, int N_Global, int K_Global, int Split_K);
+
+/*
  * SpMM_SplitK_API with the launch shape given by the caller instead of the planner
  * (for tuning a table of plans on the target machine, and for tests).  Returns
  * hipErrorInvalidValue when the shape does not fit (Waves above 8, or 4 for N = 64;
