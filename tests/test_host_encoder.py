@@ -252,3 +252,17 @@ def test_split_suggestion_follows_the_weights_density(spmm):
             assert (S, p["mode"], p["waves"], p["stage_b"]) == same_split[0]  # the densest-first table that holds this Split_K
     assert spmm.SpMM_SuggestSplitK_Bytes(1024, 24, 1024, 100) == 1
     assert spmm.SpMM_SuggestSplitK_Bytes(1000, 16, 1024, 100) == 1
+
+
+def test_where_the_slabs_are_added_up(spmm):
+    """SpMM_PlanReductionInLaunch: nothing to add with one batch; a K-splitting call adds few batches up
+    inside its launch and leaves many (or many tokens' worth) to the reduction kernel; the row-sharing
+    layout always uses the kernel; shapes the kernels do not take are refused."""
+    assert spmm.SpMM_PlanReductionInLaunch(7168, 16, 7168, 1) is False
+    assert spmm.SpMM_PlanLaunch(7168, 16, 7168, 4)["mode"] == 1 and spmm.SpMM_PlanReductionInLaunch(7168, 16, 7168, 4) is True
+    assert spmm.SpMM_PlanLaunch(4096, 64, 4096, 8)["mode"] == 1 and spmm.SpMM_PlanReductionInLaunch(4096, 64, 4096, 8) is False
+    assert spmm.SpMM_PlanLaunch(2048, 16, 8192, 16)["mode"] == 1 and spmm.SpMM_PlanReductionInLaunch(2048, 16, 8192, 16) is False
+    assert spmm.SpMM_PlanLaunch(36864, 16, 9216, 6)["mode"] == 0 and spmm.SpMM_PlanReductionInLaunch(36864, 16, 9216, 6) is False
+    for M, N, K, S in ((1000, 16, 1024, 2), (1024, 12, 1024, 2), (1024, 16, 1000, 2), (1024, 16, 1024, 0)):
+        with pytest.raises(spmm.SpMMError):
+            spmm.SpMM_PlanReductionInLaunch(M, N, K, S)
