@@ -226,7 +226,7 @@ def test_split_suggestion_follows_the_weights_density(spmm):
         """(M, K, N) -> rows in file order: the shape's measured best first, then rows for other given Split_K."""
         rows = {}
         for ln in open(os.path.join(ROOT, "graphneuralnetproj_amd", "csrc", name)):
-            m = re.match(r"\s*\{(\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+)\}", ln)
+            m = re.match(r"\s*\{(\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+)(?:, [01])?\}", ln)  # (an eighth value: reduction kernel)
             if m:
                 M, K, N, S, mode, waves, stage = map(int, m.groups())
                 rows.setdefault((M, K, N), []).append((S, mode, waves, stage))
