@@ -24,6 +24,8 @@ def test_host_code_is_clean_under_asan_and_ubsan(tmp_path):
          os.path.join(ROOT, "tests", "support", "host_sanitize.cpp")]
         + [os.path.join(CSRC, f) for f in ("tiled_csl_encode.cpp", "a24_pack.cpp", "launch_plan.cpp", "synth.cpp")],
         capture_output=True, text=True)
+    if build.returncode != 0 and ("asan" in build.stderr or "ubsan" in build.stderr) and "error:" not in build.stderr:
+        pytest.skip("this toolchain has no sanitizer runtime to link")
     assert build.returncode == 0, build.stderr[-2000:]
     run = subprocess.run([str(exe), str(tmp_path)], capture_output=True, text=True, timeout=300)
     assert run.returncode == 0, (run.stdout[-2000:], run.stderr[-4000:])
@@ -43,6 +45,8 @@ def test_counter_pages_are_race_free_under_tsan(tmp_path):
         ["g++", "-std=c++17", "-O1", "-g", "-fsanitize=thread", "-pthread", "-I", CSRC, "-o", str(exe),
          os.path.join(ROOT, "tests", "support", "counter_pages_threads.cpp"), os.path.join(CSRC, "counter_pages.cpp")],
         capture_output=True, text=True)
+    if build.returncode != 0 and "tsan" in build.stderr and "error:" not in build.stderr:
+        pytest.skip("this toolchain has no ThreadSanitizer runtime to link")
     assert build.returncode == 0, build.stderr[-2000:]
     run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300)
     if "unexpected memory mapping" in run.stderr:
