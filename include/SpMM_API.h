@@ -77,8 +77,9 @@ SPMM_EXPORT int InitSparseMatrixA_API_NoReorder(const uint16_t* A_h, int M, int 
  *   Split_K  > 1: batch b of ceil((K/64)/Split_K) column tiles writes fp16 partial
  *                 sums to Reduction_Workspace[b*M*N ..), then C = fp16(sum in fp32), added
  *                 up in batch order either by the last workgroup of the same launch to
- *                 finish a tile row (launch shape "mode 1", M <= 524288) or by a second
- *                 kernel (same bits either way).
+ *                 finish a tile row (launch shape "mode 1" with few batches, M <= 524288) or
+ *                 by a second kernel (same bits either way; the planner takes the cheaper,
+ *                 SpMM_PlanReductionInLaunch tells which).
  *                 Reduction_Workspace must hold Split_K*M*N fp16 values and may be
  *                 shared by successive calls on one stream.
  * Accumulation is fp32.  Returns the hipError_t value: 0 on success;
